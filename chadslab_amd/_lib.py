@@ -1,0 +1,61 @@
+"""ctypes binding of libchadq.so (the C ABI declared in include/chadq.h).
+
+The library is the only compute path: if it is missing or fails to load, importing an operator raises.
+There is no CPU or PyTorch fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_int, c_int64, c_void_p
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libchadq.so"
+
+# name -> (restype, argtypes); mirrors include/chadq.h one to one
+SIGNATURES = {
+    "chadq_version": (c_int, []),
+    "chadq_last_error": (c_char_p, []),
+    "chadq_arch": (c_char_p, []),
+    "chadq_unpack_i4": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "chadq_pack_i4": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "chadq_dequant_i4g32": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "chadq_dequant_i8row": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "chadq_gemv_i4g32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "chadq_gemv_i8row": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "chadq_gemm_i4g32_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "chadq_gemm_i8row_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+}
+
+_STATUS_EXC = {-1: ValueError, -2: ValueError, -3: ValueError, -4: ValueError, -5: RuntimeError, -6: RuntimeError}
+
+_lib = None
+
+
+class ChadqError(RuntimeError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Loads libchadq.so once and attaches the signatures; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise ChadqError(
+            "%s not found: build it with `python -m chadslab_amd.build` (there is no fallback path)" % LIB_PATH
+        )
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is missing
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    """Turns a negative status into a Python exception carrying the library's message."""
+    if rc == 0:
+        return
+    msg = load().chadq_last_error().decode("utf-8", "replace")
+    raise _STATUS_EXC.get(rc, RuntimeError)("%s failed (%d): %s" % (what, rc, msg))

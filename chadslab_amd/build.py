@@ -1,0 +1,63 @@
+"""Builds chadslab_amd/libchadq.so from csrc/*.hip with hipcc for gfx950 (cross-compiles without a GPU).
+
+Run as `python -m chadslab_amd.build` or through __graft_entry__.build().  The library is kept in-tree,
+next to this file; nothing is installed.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG = Path(__file__).resolve().parent
+CSRC = PKG / "csrc"
+OBJ = PKG / "csrc" / "_obj"
+LIB = PKG / "libchadq.so"
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# -packed-fp32-ops: keep the compiler from forming packed fp32 arithmetic (v_pk_*_f32)
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-Wall", "-Wno-unused-function",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _run(cmd):
+    p = subprocess.run(cmd, capture_output=True, text=True)
+    # the host pass does not know the packed-fp32 feature and says so on every file: drop that line
+    err = "\n".join(l for l in p.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if p.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s\n%s" % (" ".join(map(str, cmd)), p.stdout, err))
+    if err.strip():
+        sys.stderr.write(err + "\n")
+
+
+def build(verbose: bool = True, save_temps: bool = False) -> Path:
+    srcs = sorted(CSRC.glob("*.hip"))
+    if not srcs:
+        raise RuntimeError("no HIP sources under %s" % CSRC)
+    OBJ.mkdir(exist_ok=True)
+    objs = [OBJ / (s.stem + ".o") for s in srcs]
+
+    def one(pair):
+        s, o = pair
+        cmd = [HIPCC, *FLAGS, "-c", str(s), "-o", str(o)]
+        if save_temps:
+            cmd += ["-save-temps=obj"]
+        _run(cmd)
+        return o
+
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
+        list(ex.map(one, zip(srcs, objs)))
+    tmp = LIB.with_suffix(".so.tmp")
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)])
+    os.replace(tmp, LIB)
+    if verbose:
+        print("built %s (%d sources)" % (LIB, len(srcs)))
+    return LIB
+
+
+if __name__ == "__main__":
+    build(save_temps="--save-temps" in sys.argv)

@@ -1,0 +1,147 @@
+// extern "C" surface of libchadq.so: argument checks, error messages, dispatch.  No allocation, no copies.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "chadq_common.h"
+
+namespace chadq {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+void clear_error() { g_err[0] = '\0'; }
+
+int hip_check(hipError_t e, const char *what) {
+    if (e == hipSuccess) return 0;
+    return fail(CHADQ_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+int check_device() {
+    static int ok_mask[64] = {0};  // 0 unknown, 1 ok, -1 wrong arch; benign race: idempotent values
+    int dev = 0;
+    CHADQ_HIP(hipGetDevice(&dev));
+    if (dev >= 0 && dev < 64 && ok_mask[dev] == 1) return 0;
+    hipDeviceProp_t prop;
+    CHADQ_HIP(hipGetDeviceProperties(&prop, dev));
+    const bool ok = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+    if (dev >= 0 && dev < 64) ok_mask[dev] = ok ? 1 : -1;
+    if (!ok) return fail(CHADQ_ERR_DEVICE, "device %d is %s; libchadq is built for gfx950 only", dev, prop.gcnArchName);
+    return 0;
+}
+
+// kernels' launch functions (one per source file)
+int unpack_i4_launch(const uint8_t *, int8_t *, int64_t, hipStream_t);
+int pack_i4_launch(const int8_t *, uint8_t *, int64_t, hipStream_t);
+int dequant_i4g32_launch(const uint8_t *, const uint16_t *, float *, int, int, hipStream_t);
+int dequant_i8row_launch(const int8_t *, const float *, float *, int, int, hipStream_t);
+int gemv_i4g32_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
+int gemv_i8row_dispatch(const float *, const int8_t *, const float *, float *, int, int, int, hipStream_t);
+int gemm_i4g32_bf16_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, uint16_t *, int, int, int,
+                             hipStream_t);
+int gemm_i8row_bf16_dispatch(const uint16_t *, const int8_t *, const float *, uint16_t *, int, int, int,
+                             hipStream_t);
+
+}  // namespace chadq
+
+using namespace chadq;
+
+#define ENTER()                     \
+    clear_error();                  \
+    {                               \
+        int _d = check_device();    \
+        if (_d != 0) return _d;     \
+    }                               \
+    hipStream_t st = (hipStream_t)stream
+
+extern "C" {
+
+int chadq_version(void) { return 100; }
+
+const char *chadq_last_error(void) { return g_err; }
+
+const char *chadq_arch(void) { return "gfx950"; }
+
+int chadq_unpack_i4(const uint8_t *wp, int8_t *q, int64_t nbytes, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(nbytes >= 0, CHADQ_ERR_SHAPE, "chadq_unpack_i4: nbytes=%lld is negative", (long long)nbytes);
+    if (nbytes == 0) return 0;
+    CHADQ_REQUIRE(wp && q, CHADQ_ERR_NULL, "chadq_unpack_i4: null pointer");
+    return unpack_i4_launch(wp, q, nbytes, st);
+}
+
+int chadq_pack_i4(const int8_t *q, uint8_t *wp, int64_t nbytes, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(nbytes >= 0, CHADQ_ERR_SHAPE, "chadq_pack_i4: nbytes=%lld is negative", (long long)nbytes);
+    if (nbytes == 0) return 0;
+    CHADQ_REQUIRE(wp && q, CHADQ_ERR_NULL, "chadq_pack_i4: null pointer");
+    return pack_i4_launch(q, wp, nbytes, st);
+}
+
+int chadq_dequant_i4g32(const uint8_t *wp, const uint16_t *scale_f16, float *w, int N, int K, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(N >= 0 && K >= 0 && K % 32 == 0, CHADQ_ERR_SHAPE, "chadq_dequant_i4g32: N=%d K=%d (K %% 32 != 0?)", N, K);
+    if (N == 0 || K == 0) return 0;
+    CHADQ_REQUIRE(wp && scale_f16 && w, CHADQ_ERR_NULL, "chadq_dequant_i4g32: null pointer");
+    CHADQ_REQUIRE(aligned16(wp) && aligned16(w), CHADQ_ERR_ALIGN, "chadq_dequant_i4g32: wp and w must be 16-byte aligned");
+    return dequant_i4g32_launch(wp, scale_f16, w, N, K, st);
+}
+
+int chadq_dequant_i8row(const int8_t *w8, const float *scale, float *w, int N, int K, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(N >= 0 && K >= 0, CHADQ_ERR_SHAPE, "chadq_dequant_i8row: N=%d K=%d", N, K);
+    if (N == 0 || K == 0) return 0;
+    CHADQ_REQUIRE(w8 && scale && w, CHADQ_ERR_NULL, "chadq_dequant_i8row: null pointer");
+    return dequant_i8row_launch(w8, scale, w, N, K, st);
+}
+
+int chadq_gemv_i4g32(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *scale_f16, float *y, int M, int N,
+                     int K, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(M >= 1 && M <= 16, CHADQ_ERR_SHAPE, "chadq_gemv_i4g32: M=%d outside [1,16] (use chadq_gemm_i4g32_bf16)", M);
+    CHADQ_REQUIRE(N >= 0 && K >= 32 && K % 32 == 0, CHADQ_ERR_SHAPE, "chadq_gemv_i4g32: N=%d K=%d (K must be a positive multiple of 32)", N, K);
+    if (N == 0) return 0;
+    CHADQ_REQUIRE(x_bf16 && wp && scale_f16 && y, CHADQ_ERR_NULL, "chadq_gemv_i4g32: null pointer");
+    CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(wp), CHADQ_ERR_ALIGN, "chadq_gemv_i4g32: x and wp must be 16-byte aligned");
+    return gemv_i4g32_dispatch(x_bf16, wp, scale_f16, y, M, N, K, st);
+}
+
+int chadq_gemv_i8row(const float *x, const int8_t *w8, const float *scale, float *y, int M, int N, int K,
+                     void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(M >= 1 && M <= 16, CHADQ_ERR_SHAPE, "chadq_gemv_i8row: M=%d outside [1,16]", M);
+    CHADQ_REQUIRE(N >= 0 && K >= 16 && K % 16 == 0, CHADQ_ERR_SHAPE, "chadq_gemv_i8row: N=%d K=%d (K must be a positive multiple of 16)", N, K);
+    if (N == 0) return 0;
+    CHADQ_REQUIRE(x && w8 && scale && y, CHADQ_ERR_NULL, "chadq_gemv_i8row: null pointer");
+    CHADQ_REQUIRE(aligned16(x) && aligned16(w8), CHADQ_ERR_ALIGN, "chadq_gemv_i8row: x and w8 must be 16-byte aligned");
+    return gemv_i8row_dispatch(x, w8, scale, y, M, N, K, st);
+}
+
+int chadq_gemm_i4g32_bf16(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *scale_f16, uint16_t *y_bf16,
+                          int M, int N, int K, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(M >= 0 && N >= 0 && K >= 32 && K % 32 == 0, CHADQ_ERR_SHAPE, "chadq_gemm_i4g32_bf16: M=%d N=%d K=%d (K must be a positive multiple of 32)", M, N, K);
+    if (M == 0 || N == 0) return 0;
+    CHADQ_REQUIRE(x_bf16 && wp && scale_f16 && y_bf16, CHADQ_ERR_NULL, "chadq_gemm_i4g32_bf16: null pointer");
+    CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(wp), CHADQ_ERR_ALIGN, "chadq_gemm_i4g32_bf16: x and wp must be 16-byte aligned");
+    return gemm_i4g32_bf16_dispatch(x_bf16, wp, scale_f16, y_bf16, M, N, K, st);
+}
+
+int chadq_gemm_i8row_bf16(const uint16_t *x_bf16, const int8_t *w8, const float *scale, uint16_t *y_bf16, int M,
+                          int N, int K, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(M >= 0 && N >= 0 && K >= 16 && K % 16 == 0, CHADQ_ERR_SHAPE, "chadq_gemm_i8row_bf16: M=%d N=%d K=%d (K must be a positive multiple of 16)", M, N, K);
+    if (M == 0 || N == 0) return 0;
+    CHADQ_REQUIRE(x_bf16 && w8 && scale && y_bf16, CHADQ_ERR_NULL, "chadq_gemm_i8row_bf16: null pointer");
+    CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(w8), CHADQ_ERR_ALIGN, "chadq_gemm_i8row_bf16: x and w8 must be 16-byte aligned");
+    return gemm_i8row_bf16_dispatch(x_bf16, w8, scale, y_bf16, M, N, K, st);
+}
+
+}  // extern "C"

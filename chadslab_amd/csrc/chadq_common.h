@@ -1,0 +1,109 @@
+// Shared device helpers and the host-side error plumbing for libchadq (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/chadq.h"
+
+namespace chadq {
+
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+constexpr int kWave = 64;
+constexpr int kGroup = 32;                  // int4 scale group along K
+constexpr uint32_t kBf16Magic = 0x43004300u;  // two bf16 128.0: OR a nibble into the low mantissa bits -> 128+u
+constexpr float kMagicBias = 136.0f;          // 128 (magic) + 8 (zero point)
+
+// ---- host side: status + thread-local message -------------------------------------------------
+int fail(int code, const char *fmt, ...);
+void clear_error();
+// 0 if `call` succeeded, else records the HIP error and returns CHADQ_ERR_HIP.
+int hip_check(hipError_t e, const char *what);
+// checks that the current device is gfx950 (cached per device)
+int check_device();
+
+#define CHADQ_HIP(call)                                  \
+    do {                                                 \
+        int _rc = ::chadq::hip_check((call), #call);     \
+        if (_rc != 0) return _rc;                        \
+    } while (0)
+
+#define CHADQ_REQUIRE(cond, code, ...)                       \
+    do {                                                     \
+        if (!(cond)) return ::chadq::fail((code), __VA_ARGS__); \
+    } while (0)
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- device side ------------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) { return __uint_as_float(lo16 << 16); }
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+    _Float16 v;
+    __builtin_memcpy(&v, &h, 2);
+    return (float)v;
+}
+
+// fp32 -> bf16 bits, round to nearest even, NaN kept quiet.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x0040u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+__device__ __forceinline__ bf16x2 as_bf16x2(uint32_t v) {
+    bf16x2 r;
+    __builtin_memcpy(&r, &v, 4);
+    return r;
+}
+
+// One 32-bit word of packed weights = 8 nibbles u0..u7 (u0 lowest).  Returns four registers of bf16
+// pairs holding 128+u: p[i] = (128+u_i , 128+u_{i+4}), i = 0..3.  Exact: 128+u <= 143 fits bf16.
+__device__ __forceinline__ void unpack8_magic(uint32_t w, uint32_t p[4]) {
+    constexpr uint32_t m = 0x000F000Fu;
+    p[0] = (w & m) | kBf16Magic;
+    p[1] = ((w >> 4) & m) | kBf16Magic;
+    p[2] = ((w >> 8) & m) | kBf16Magic;
+    p[3] = ((w >> 12) & m) | kBf16Magic;
+}
+
+// Eight consecutive bf16 activations in four registers a[0..3] = (x0,x1),(x2,x3),(x4,x5),(x6,x7) are
+// rearranged to match unpack8_magic's pairing: o[i] = (x_i, x_{i+4}).
+__device__ __forceinline__ void pair_x8(const uint32_t a[4], uint32_t o[4]) {
+    o[0] = __builtin_amdgcn_perm(a[2], a[0], 0x05040100u);
+    o[1] = __builtin_amdgcn_perm(a[2], a[0], 0x07060302u);
+    o[2] = __builtin_amdgcn_perm(a[3], a[1], 0x05040100u);
+    o[3] = __builtin_amdgcn_perm(a[3], a[1], 0x07060302u);
+}
+
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(as_bf16x2(a), as_bf16x2(b), c, false);
+}
+
+// data-parallel-primitive move: value of `v` from the lane selected by CTRL, 0 where masked off
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, false));
+}
+
+// Sum over the 64 lanes of a wavefront; the total is valid in lane 63 only.
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+    v += dpp_f32<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+    v += dpp_f32<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+    v += dpp_f32<0x141, 0xF>(v);  // row_half_mirror
+    v += dpp_f32<0x140, 0xF>(v);  // row_mirror: every lane of a 16-lane row now holds the row sum
+    v += dpp_f32<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
+    v += dpp_f32<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
+    return v;
+}
+
+__device__ __forceinline__ u32x4 load_nt_b128(const void *p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+}
+
+}  // namespace chadq

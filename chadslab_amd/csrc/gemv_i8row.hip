@@ -1,0 +1,145 @@
+// Decode GEMV on int8 weights with one fp32 scale per output row:  y[m,n] = s[n] * sum_k x[m,k] * W[n,k].
+//
+// HBM-bound stream of W.  A wavefront owns whole rows; one 128-bit load per lane = 16 weights, a wave-wide
+// load = 1024 consecutive k (1 KiB contiguous).  All loads of a wave are issued first; the fp32 activations
+// of the lane's k positions are read once and stay in registers.  Signed bytes are flipped to unsigned
+// (w ^ 0x80 = w + 128) so that v_cvt_f32_ubyteN converts them in one instruction; the accumulator starts
+// at -128 * sum(x) to take the offset back out.  DPP adds fold the 64 partial sums; no LDS.
+#include "chadq_common.h"
+
+namespace chadq {
+
+__device__ __forceinline__ float ubyte_to_f32(uint32_t v, int i) { return (float)((v >> (8 * i)) & 0xFFu); }
+
+template <int CH, int R, int MB>
+__global__ __launch_bounds__(256) void gemv_i8row_rows_kernel(const float *__restrict__ x,
+                                                              const int8_t *__restrict__ w8,
+                                                              const float *__restrict__ sc, float *__restrict__ y,
+                                                              int N, int K) {
+    const int lane = threadIdx.x & 63;
+    const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int row0 = gw * R;
+    if (row0 >= N) return;
+
+    u32x4 w[R][CH];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int row = row0 + r;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int k0 = c * 1024 + lane * 16;
+            const bool ok = (row < N) && (k0 < K);
+            w[r][c] = ok ? load_nt_b128(w8 + (size_t)row * K + k0) : u32x4{0, 0, 0, 0};
+        }
+    }
+
+    float xs[MB][CH][16];
+    float bias[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        float sum = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int k0 = c * 1024 + lane * 16;
+            const bool ok = k0 < K;
+            const f32x4 *xp = reinterpret_cast<const f32x4 *>(x + (size_t)m * K + k0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const f32x4 v = ok ? xp[i] : f32x4{0.f, 0.f, 0.f, 0.f};
+                xs[m][c][4 * i + 0] = v.x;
+                xs[m][c][4 * i + 1] = v.y;
+                xs[m][c][4 * i + 2] = v.z;
+                xs[m][c][4 * i + 3] = v.w;
+                sum += (v.x + v.y) + (v.z + v.w);
+            }
+        }
+        bias[m] = -128.f * sum;
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        float acc[MB];
+#pragma unroll
+        for (int m = 0; m < MB; ++m) acc[m] = bias[m];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const uint32_t ww[4] = {w[r][c].x ^ 0x80808080u, w[r][c].y ^ 0x80808080u, w[r][c].z ^ 0x80808080u,
+                                    w[r][c].w ^ 0x80808080u};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float f = ubyte_to_f32(ww[j], i);
+#pragma unroll
+                    for (int m = 0; m < MB; ++m) acc[m] = __builtin_fmaf(xs[m][c][4 * j + i], f, acc[m]);
+                }
+        }
+        const int row = row0 + r;
+        const float s = (row < N) ? sc[row] : 0.f;
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            const float t = wave_sum_to_lane63(acc[m]);
+            if (lane == 63 && row < N) y[(size_t)m * N + row] = t * s;
+        }
+    }
+}
+
+// Any K % 16 == 0 and any M; one wave per row, 1024-wide chunks streamed in a loop.
+__global__ __launch_bounds__(256) void gemv_i8row_generic_kernel(const float *__restrict__ x,
+                                                                 const int8_t *__restrict__ w8,
+                                                                 const float *__restrict__ sc,
+                                                                 float *__restrict__ y, int M, int N, int K) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const float s = sc[row];
+    for (int m = 0; m < M; ++m) {
+        float acc = 0.f;
+        for (int k0 = lane * 16; k0 < K; k0 += 1024) {
+            const u32x4 wv = *reinterpret_cast<const u32x4 *>(w8 + (size_t)row * K + k0);
+            const uint32_t ww[4] = {wv.x ^ 0x80808080u, wv.y ^ 0x80808080u, wv.z ^ 0x80808080u, wv.w ^ 0x80808080u};
+            const f32x4 *xp = reinterpret_cast<const f32x4 *>(x + (size_t)m * K + k0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f32x4 v = xp[j];
+                acc = __builtin_fmaf(v.x, ubyte_to_f32(ww[j], 0) - 128.f, acc);
+                acc = __builtin_fmaf(v.y, ubyte_to_f32(ww[j], 1) - 128.f, acc);
+                acc = __builtin_fmaf(v.z, ubyte_to_f32(ww[j], 2) - 128.f, acc);
+                acc = __builtin_fmaf(v.w, ubyte_to_f32(ww[j], 3) - 128.f, acc);
+            }
+        }
+        const float t = wave_sum_to_lane63(acc);
+        if (lane == 63) y[(size_t)m * N + row] = t * s;
+    }
+}
+
+template <int CH, int R, int MB>
+static void launch_rows8(const float *x, const int8_t *w8, const float *sc, float *y, int N, int K, hipStream_t st) {
+    const int waves = (N + R - 1) / R;
+    hipLaunchKernelGGL((gemv_i8row_rows_kernel<CH, R, MB>), dim3((waves + 3) / 4), dim3(256), 0, st, x, w8, sc, y, N, K);
+}
+
+int gemv_i8row_dispatch(const float *x, const int8_t *w8, const float *sc, float *y, int M, int N, int K,
+                        hipStream_t st) {
+    if (K <= 2048) {
+        const bool big = N >= 8192;
+        for (int m0 = 0; m0 < M;) {
+            const float *xm = x + (size_t)m0 * K;
+            float *ym = y + (size_t)m0 * N;
+            const int mb = (M - m0 >= 2) ? 2 : 1;
+            if (K <= 1024) {
+                if (mb == 2) big ? launch_rows8<1, 8, 2>(xm, w8, sc, ym, N, K, st) : launch_rows8<1, 2, 2>(xm, w8, sc, ym, N, K, st);
+                else big ? launch_rows8<1, 8, 1>(xm, w8, sc, ym, N, K, st) : launch_rows8<1, 2, 1>(xm, w8, sc, ym, N, K, st);
+            } else {
+                if (mb == 2) big ? launch_rows8<2, 4, 2>(xm, w8, sc, ym, N, K, st) : launch_rows8<2, 1, 2>(xm, w8, sc, ym, N, K, st);
+                else big ? launch_rows8<2, 4, 1>(xm, w8, sc, ym, N, K, st) : launch_rows8<2, 1, 1>(xm, w8, sc, ym, N, K, st);
+            }
+            m0 += mb;
+        }
+    } else {
+        hipLaunchKernelGGL(gemv_i8row_generic_kernel, dim3((N + 3) / 4), dim3(256), 0, st, x, w8, sc, y, M, N, K);
+    }
+    return hip_check(hipGetLastError(), "gemv_i8row launch");
+}
+
+}  // namespace chadq

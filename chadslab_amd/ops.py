@@ -1,0 +1,127 @@
+"""Operator entry points: what a numpy-style LLM runtime's quantized `x @ dequant(W).T` call sites bind to.
+
+Every function runs hand-written HIP kernels from libchadq.so through its C ABI (chadslab_amd/_lib.py) on
+torch's current stream.  torch is used for device memory and streams only.  Nothing here computes on the
+CPU: tensors must already be on the GPU, and a missing library raises.
+"""
+from __future__ import annotations
+
+from typing import Optional, Union
+
+import torch
+
+from . import _lib
+from .formats import QWeightInt4G32, QWeightInt8
+
+QWeight = Union[QWeightInt4G32, QWeightInt8]
+GEMV_MAX_M = 16  # decode batch sizes served by the bandwidth kernel
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, name: str, dtype: torch.dtype) -> torch.Tensor:
+    if not t.is_cuda:
+        raise ValueError("%s must be a GPU tensor (there is no CPU path)" % name)
+    if t.dtype != dtype:
+        raise ValueError("%s must be %s, got %s" % (name, dtype, t.dtype))
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def unpack_int4(packed: torch.Tensor) -> torch.Tensor:
+    """uint8 [..., K/2] -> int8 [..., K] in [-8,7] (low nibble = even k)."""
+    p = _dev(packed, "packed", torch.uint8)
+    out = torch.empty(*p.shape[:-1], p.shape[-1] * 2, dtype=torch.int8, device=p.device)
+    _lib.check(_lib.load().chadq_unpack_i4(p.data_ptr(), out.data_ptr(), p.numel(), _stream()), "chadq_unpack_i4")
+    return out
+
+
+def pack_int4(q: torch.Tensor) -> torch.Tensor:
+    """int8 [..., K] in [-8,7] -> uint8 [..., K/2]; inverse of unpack_int4."""
+    q = _dev(q, "q", torch.int8)
+    if q.shape[-1] % 2:
+        raise ValueError("K must be even")
+    out = torch.empty(*q.shape[:-1], q.shape[-1] // 2, dtype=torch.uint8, device=q.device)
+    _lib.check(_lib.load().chadq_pack_i4(q.data_ptr(), out.data_ptr(), out.numel(), _stream()), "chadq_pack_i4")
+    return out
+
+
+def dequantize(qw: QWeight) -> torch.Tensor:
+    """fp32 [N,K] dequantised weights (exact)."""
+    lib = _lib.load()
+    if isinstance(qw, QWeightInt4G32):
+        p, s = _dev(qw.packed, "packed", torch.uint8), _dev(qw.scale, "scale", torch.float16)
+        out = torch.empty(qw.N, qw.K, dtype=torch.float32, device=p.device)
+        _lib.check(lib.chadq_dequant_i4g32(p.data_ptr(), s.data_ptr(), out.data_ptr(), qw.N, qw.K, _stream()),
+                   "chadq_dequant_i4g32")
+        return out
+    if isinstance(qw, QWeightInt8):
+        w, s = _dev(qw.w, "w", torch.int8), _dev(qw.scale, "scale", torch.float32)
+        out = torch.empty(qw.N, qw.K, dtype=torch.float32, device=w.device)
+        _lib.check(lib.chadq_dequant_i8row(w.data_ptr(), s.data_ptr(), out.data_ptr(), qw.N, qw.K, _stream()),
+                   "chadq_dequant_i8row")
+        return out
+    raise TypeError("unknown weight container %r" % type(qw))
+
+
+def qgemv(x: torch.Tensor, qw: QWeight, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Decode product, fp32 out [M,N], M <= 16.  x is bf16 [M,K] for int4 weights, fp32 [M,K] for int8 weights."""
+    lib = _lib.load()
+    if x.dim() != 2 or x.shape[1] != qw.K:
+        raise ValueError("x must be [M,%d], got %s" % (qw.K, tuple(x.shape)))
+    m = x.shape[0]
+    if isinstance(qw, QWeightInt4G32):
+        x = _dev(x, "x", torch.bfloat16)
+        p, s = _dev(qw.packed, "packed", torch.uint8), _dev(qw.scale, "scale", torch.float16)
+        y = out if out is not None else torch.empty(m, qw.N, dtype=torch.float32, device=x.device)
+        _lib.check(lib.chadq_gemv_i4g32(x.data_ptr(), p.data_ptr(), s.data_ptr(), y.data_ptr(), m, qw.N, qw.K,
+                                        _stream()), "chadq_gemv_i4g32")
+        return y
+    if isinstance(qw, QWeightInt8):
+        x = _dev(x, "x", torch.float32)
+        w, s = _dev(qw.w, "w", torch.int8), _dev(qw.scale, "scale", torch.float32)
+        y = out if out is not None else torch.empty(m, qw.N, dtype=torch.float32, device=x.device)
+        _lib.check(lib.chadq_gemv_i8row(x.data_ptr(), w.data_ptr(), s.data_ptr(), y.data_ptr(), m, qw.N, qw.K,
+                                        _stream()), "chadq_gemv_i8row")
+        return y
+    raise TypeError("unknown weight container %r" % type(qw))
+
+
+def qgemm(x: torch.Tensor, qw: QWeight, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Prefill product on the matrix cores: x bf16 [M,K] -> bf16 [M,N], fp32 accumulate."""
+    lib = _lib.load()
+    if x.dim() != 2 or x.shape[1] != qw.K:
+        raise ValueError("x must be [M,%d], got %s" % (qw.K, tuple(x.shape)))
+    x = _dev(x, "x", torch.bfloat16)
+    m = x.shape[0]
+    y = out if out is not None else torch.empty(m, qw.N, dtype=torch.bfloat16, device=x.device)
+    if isinstance(qw, QWeightInt4G32):
+        p, s = _dev(qw.packed, "packed", torch.uint8), _dev(qw.scale, "scale", torch.float16)
+        _lib.check(lib.chadq_gemm_i4g32_bf16(x.data_ptr(), p.data_ptr(), s.data_ptr(), y.data_ptr(), m, qw.N, qw.K,
+                                             _stream()), "chadq_gemm_i4g32_bf16")
+    elif isinstance(qw, QWeightInt8):
+        w, s = _dev(qw.w, "w", torch.int8), _dev(qw.scale, "scale", torch.float32)
+        _lib.check(lib.chadq_gemm_i8row_bf16(x.data_ptr(), w.data_ptr(), s.data_ptr(), y.data_ptr(), m, qw.N, qw.K,
+                                             _stream()), "chadq_gemm_i8row_bf16")
+    else:
+        raise TypeError("unknown weight container %r" % type(qw))
+    return y
+
+
+def qlinear(x: torch.Tensor, qw: QWeight, *, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """y = x @ dequant(W).T over the last axis of x.
+
+    Up to 16 rows go to the bandwidth-bound GEMV (fp32 result); more rows go to the MFMA GEMM (bf16 result).
+    out_dtype picks the result type; asking for the other type than the kernel's native one casts.
+    """
+    lead, k = x.shape[:-1], x.shape[-1]
+    x2 = x.reshape(-1, k)
+    m = x2.shape[0]
+    use_gemv = m <= GEMV_MAX_M and not (isinstance(qw, QWeightInt8) and x2.dtype == torch.bfloat16)
+    if isinstance(qw, QWeightInt8) and x2.dtype == torch.float32 and not use_gemv:
+        raise ValueError("int8 weights with fp32 activations are served for at most %d rows" % GEMV_MAX_M)
+    y = qgemv(x2, qw) if use_gemv else qgemm(x2, qw)
+    if out_dtype is not None and y.dtype != out_dtype:
+        y = y.to(out_dtype)
+    return y.reshape(*lead, qw.N)

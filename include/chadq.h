@@ -1,0 +1,107 @@
+/*
+ * chadq.h — C ABI of libchadq.so: quantized-weight matrix products on MI355X (gfx950).
+ *
+ * This is the drop-in boundary for one path only: unpacking packed int8/int4 weights
+ * with their scales, fused dequantisation, and the GEMV (decode) / GEMM (prefill, MoE
+ * expert) products on them.
+ *
+ * Reference interface replaced: none exists.  The reference snapshot
+ * (happycube/chadslab) has no numpy-gemma/ or reclank/ runtime, no op table, no IR
+ * interpreter and no FFI layer (its top level is README, ancientARMS/, hsv2.c, kaggle/,
+ * m++/, m6502/, notebooks/, nv-fansetup/, ppmproc.cxx, sand/, talks/), so no entry
+ * point below can cite a reference file:line.  Each one instead cites the closed form
+ * of the benchmark configuration it computes; the Python operator layer in
+ * chadslab_amd/ops.py is what a numpy runtime's `x @ dequant(W).T` call sites would
+ * bind to.
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer owned by the caller.  The library allocates no
+ *    device memory and does no host<->device copies.
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Launches are
+ *    asynchronous on that stream.
+ *  - Return value: 0 on success, a negative chadq_status otherwise; the message for
+ *    the calling thread's last failure is chadq_last_error().  No C++ exception crosses
+ *    this boundary.
+ *  - Formats (this build's choices where the configuration text is silent):
+ *      int8 per-row : W int8 [N,K] row-major, scale fp32 [N];  w = W[n,k] * scale[n]
+ *      int4 group-32: Wp uint8 [N,K/2] row-major, byte j of a row = (u[2j]) | (u[2j+1] << 4),
+ *                     u = q + 8 in [0,15]; scale fp16 [N,K/32]; w = (u - 8) * scale[n,k/32]
+ *      bf16 / fp16 values travel as uint16_t bit patterns.
+ */
+#ifndef CHADQ_H
+#define CHADQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum chadq_status {
+    CHADQ_OK = 0,
+    CHADQ_ERR_NULL = -1,      /* a required pointer is NULL */
+    CHADQ_ERR_SHAPE = -2,     /* a dimension is non-positive or breaks a divisibility rule */
+    CHADQ_ERR_ALIGN = -3,     /* a pointer is not aligned as the entry point requires */
+    CHADQ_ERR_WORKSPACE = -4, /* workspace missing or too small */
+    CHADQ_ERR_HIP = -5,       /* a HIP call failed; the message names it */
+    CHADQ_ERR_DEVICE = -6     /* the current device is not gfx950 */
+} chadq_status;
+
+/* Library version, major*10000 + minor*100 + patch. */
+int chadq_version(void);
+
+/* Message for the last failure on the calling thread ("" if none). Never NULL. */
+const char *chadq_last_error(void);
+
+/* Name of the gfx architecture the kernels were compiled for ("gfx950"). */
+const char *chadq_arch(void);
+
+/* ---- unpack / dequantise (parity and tooling entry points) -------------------------- */
+
+/* nbytes packed bytes -> 2*nbytes int8 values in [-8,7] (low nibble first). Bit-exact. */
+int chadq_unpack_i4(const uint8_t *wp, int8_t *q, int64_t nbytes, void *stream);
+
+/* 2*nbytes int8 values in [-8,7] -> nbytes packed bytes; inverse of chadq_unpack_i4. */
+int chadq_pack_i4(const int8_t *q, uint8_t *wp, int64_t nbytes, void *stream);
+
+/* w[n,k] = (u[n,k]-8) * float(scale[n,k/32]) as fp32 [N,K]; exact (no rounding occurs). K%32==0. */
+int chadq_dequant_i4g32(const uint8_t *wp, const uint16_t *scale_f16, float *w, int N, int K, void *stream);
+
+/* w[n,k] = W[n,k] * scale[n] as fp32 [N,K]. */
+int chadq_dequant_i8row(const int8_t *w8, const float *scale, float *w, int N, int K, void *stream);
+
+/* ---- decode GEMV (benchmark configs 0 and 1) ----------------------------------------- */
+
+/*
+ * y[m,n] = sum_g float(scale[n,g]) * sum_{k in g} x[m,k] * (u[n,k]-8)      (config 1)
+ * x bf16 [M,K], y fp32 [M,N], 1 <= M <= 16, K % 32 == 0.  wp and x 16-byte aligned.
+ * HBM-bound: each packed weight byte and each scale is read once for all M rows.
+ */
+int chadq_gemv_i4g32(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *scale_f16, float *y, int M, int N,
+                     int K, void *stream);
+
+/*
+ * y[m,n] = scale[n] * sum_k x[m,k] * W[n,k]                                 (config 0)
+ * x fp32 [M,K], W int8 [N,K], scale fp32 [N], y fp32 [M,N], 1 <= M <= 16, K % 16 == 0.
+ */
+int chadq_gemv_i8row(const float *x, const int8_t *w8, const float *scale, float *y, int M, int N, int K,
+                     void *stream);
+
+/* ---- prefill dequant-GEMM (benchmark config 2) ---------------------------------------- */
+
+/*
+ * y[m,n] = bf16_rne( sum_k x[m,k] * w[n,k] ), w as in chadq_dequant_i4g32 rounded to bf16
+ * for the MFMA, fp32 accumulate.  x bf16 [M,K], y bf16 [M,N].  K % 32 == 0, any M >= 1.
+ */
+int chadq_gemm_i4g32_bf16(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *scale_f16, uint16_t *y_bf16,
+                          int M, int N, int K, void *stream);
+
+/* Same with int8 weights and one fp32 scale per output row (scale applied in fp32 after the MFMA). */
+int chadq_gemm_i8row_bf16(const uint16_t *x_bf16, const int8_t *w8, const float *scale, uint16_t *y_bf16, int M,
+                          int N, int K, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CHADQ_H */

@@ -1,0 +1,219 @@
+"""CPU oracle for the quantized-weight matrix-product path.  TEST INFRASTRUCTURE ONLY.
+
+This module is the checker: only tests/, __graft_entry__.smoke() and the
+cpu_baseline leg of bench.py may import it.  Nothing under chadslab_amd/ does.
+
+What it restates
+----------------
+The reference snapshot (happycube/chadslab) holds no quantized-matmul code: no
+numpy-gemma/, no reclank/, no int4/int8 unpack, dequant, GEMV or GEMM (its
+top level is README, ancientARMS/, hsv2.c, kaggle/, m++/, m6502/, notebooks/,
+nv-fansetup/, ppmproc.cxx, sand/, talks/).  So there is no reference file:line
+for any function below.  Each one restates, in the plainest numpy a CPU runtime
+would use, the closed form the benchmark configuration text gives:
+
+  config 0  y = x . (W . s)^T, W int8 [N,K], s fp32 [N] per output row
+  config 1  W int4 packed 2 per byte, group 32 along K, fp16 scale per group,
+            symmetric (zero-point 8), fp32 out
+  config 2  same weights, fp32 accumulate, bf16 out
+  config 3  softmax top-2 routing, SiLU-gated experts, bf16 out
+  config 4  Gemma-2B-shaped decoder step
+
+Layout choices that the configuration text leaves open are this build's own
+and are stated where they are made (nibble order, top-2 renormalisation, the
+gate/up reading, the rounding of the MoE intermediate).  PARITY UNPINNED
+against the reference for those choices: nothing in the snapshot can pin them.
+What pins every function instead (tests/test_oracle_*.py): exhaustive
+enumeration for pack/unpack, triple-loop brute force on tiny shapes, special
+cases with exact answers, library cross-checks (scipy softmax, torch silu,
+torch bf16 rounding, torch matmul), int64 brute force for the exact-integer
+accumulation case, and the independent scalar C twin in chadq_oracle.c.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+GROUP = 32          # int4 scale group length along K
+ZERO_POINT = 8      # stored nibble u = q + 8, q in [-8, 7]
+
+
+# --------------------------------------------------------------------------- bf16
+def bf16_to_f32(bits: np.ndarray) -> np.ndarray:
+    """uint16 bf16 bit patterns -> float32 (exact: bf16 is the top half of fp32)."""
+    bits = np.asarray(bits, dtype=np.uint16)
+    return (bits.astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def f32_to_bf16(x: np.ndarray) -> np.ndarray:
+    """float32 -> bf16 bit patterns, round-to-nearest-even; NaN stays a quiet NaN."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32)
+    lsb = (u >> np.uint32(16)) & np.uint32(1)
+    rounded = ((u + np.uint32(0x7FFF) + lsb) >> np.uint32(16)).astype(np.uint16)
+    nan = np.isnan(x)
+    if nan.any():
+        rounded = np.where(nan, ((u >> np.uint32(16)) | np.uint32(0x0040)).astype(np.uint16), rounded)
+    return rounded
+
+
+# --------------------------------------------------------------------------- int4 pack
+def pack_int4(q: np.ndarray) -> np.ndarray:
+    """q int8 [N,K] with values in [-8,7] -> uint8 [N,K/2].
+
+    BUILD CHOICE (nibble order): byte j of a row holds k=2j in its low nibble and
+    k=2j+1 in its high nibble, K contiguous; stored nibble is q+8.
+    """
+    q = np.asarray(q)
+    if q.ndim != 2 or q.shape[1] % 2:
+        raise ValueError("pack_int4 wants [N,K] with even K")
+    if q.min(initial=0) < -8 or q.max(initial=0) > 7:
+        raise ValueError("int4 values must lie in [-8,7]")
+    u = (q.astype(np.int16) + ZERO_POINT).astype(np.uint8)
+    return (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8)
+
+
+def unpack_int4(wp: np.ndarray) -> np.ndarray:
+    """uint8 [N,K/2] -> int8 [N,K] in [-8,7]; inverse of pack_int4."""
+    wp = np.asarray(wp, dtype=np.uint8)
+    n, kh = wp.shape
+    q = np.empty((n, kh * 2), dtype=np.int8)
+    q[:, 0::2] = (wp & 0x0F).astype(np.int8) - ZERO_POINT
+    q[:, 1::2] = (wp >> 4).astype(np.int8) - ZERO_POINT
+    return q
+
+
+# --------------------------------------------------------------------------- dequant
+def dequant_int8(w: np.ndarray, scale: np.ndarray) -> np.ndarray:
+    """W int8 [N,K], scale fp32 [N] -> fp32 [N,K] = W[n,k] * s[n]."""
+    return w.astype(np.float32) * np.asarray(scale, dtype=np.float32)[:, None]
+
+
+def dequant_int4g32(wp: np.ndarray, scale_f16: np.ndarray) -> np.ndarray:
+    """packed uint8 [N,K/2], scale fp16 [N,K/32] -> fp32 [N,K] = (u-8) * float(s[n,k//32]).
+
+    The product is exact in fp32 (4-bit integer times 11-bit significand).
+    """
+    q = unpack_int4(wp).astype(np.float32)
+    s = np.asarray(scale_f16, dtype=np.float16).astype(np.float32)
+    if s.shape != (q.shape[0], q.shape[1] // GROUP):
+        raise ValueError("scale must be [N, K/32]")
+    return q * np.repeat(s, GROUP, axis=1)
+
+
+# --------------------------------------------------------------------------- GEMV / GEMM
+def qgemv_int8(x: np.ndarray, w: np.ndarray, scale: np.ndarray) -> np.ndarray:
+    """Config 0 as a numpy runtime computes it: y = x . (W . s)^T, all fp32.  x [M,K] -> [M,N]."""
+    return np.asarray(x, dtype=np.float32) @ dequant_int8(w, scale).T
+
+
+def qgemv_int8_f64(x, w, scale) -> np.ndarray:
+    """Ground truth for config 0 in float64."""
+    wd = w.astype(np.float64) * np.asarray(scale, dtype=np.float32).astype(np.float64)[:, None]
+    return np.asarray(x, dtype=np.float32).astype(np.float64) @ wd.T
+
+
+def qgemm_int4g32_f64(x_bf16: np.ndarray, wp: np.ndarray, scale_f16: np.ndarray) -> np.ndarray:
+    """Ground truth: float64 product of the bf16 activations with the exactly dequantised weights."""
+    x = bf16_to_f32(x_bf16).astype(np.float64)
+    return x @ dequant_int4g32(wp, scale_f16).astype(np.float64).T
+
+
+def qgemv_int4g32(x_bf16: np.ndarray, wp: np.ndarray, scale_f16: np.ndarray) -> np.ndarray:
+    """Configs 1: x bf16 bits [M,K] -> fp32 [M,N]; dequantise to fp32, then an fp32 matmul."""
+    return bf16_to_f32(x_bf16) @ dequant_int4g32(wp, scale_f16).T
+
+
+def qgemm_int4g32_bf16(x_bf16, wp, scale_f16) -> np.ndarray:
+    """Config 2: fp32 accumulate, bf16 (RNE) out.  Returns bf16 bit patterns [M,N]."""
+    return f32_to_bf16(qgemv_int4g32(x_bf16, wp, scale_f16))
+
+
+def qgemm_int8_bf16(x_bf16, w, scale) -> np.ndarray:
+    """Config 2's int8 variant: x bf16 [M,K], W int8 per-row scale, bf16 (RNE) out."""
+    return f32_to_bf16(bf16_to_f32(x_bf16) @ dequant_int8(w, scale).T)
+
+
+def qgemm_int8_f64(x_bf16, w, scale) -> np.ndarray:
+    wd = w.astype(np.float64) * np.asarray(scale, dtype=np.float32).astype(np.float64)[:, None]
+    return bf16_to_f32(x_bf16).astype(np.float64) @ wd.T
+
+
+# --------------------------------------------------------------------------- MoE
+def softmax(logits: np.ndarray) -> np.ndarray:
+    z = np.asarray(logits, dtype=np.float32)
+    z = z - z.max(axis=-1, keepdims=True)
+    e = np.exp(z)
+    return (e / e.sum(axis=-1, keepdims=True)).astype(np.float32)
+
+
+def moe_route(logits: np.ndarray, top_k: int = 2, renorm: bool = True):
+    """softmax over experts, then the top_k largest probabilities per token.
+
+    Ties go to the lower expert index (a stable sort of -p).  BUILD CHOICE:
+    renorm=True divides the selected weights by their sum (they then add to 1).
+    Returns (idx int32 [T,top_k], w fp32 [T,top_k]).
+    """
+    p = softmax(logits)
+    idx = np.argsort(-p, axis=-1, kind="stable")[:, :top_k].astype(np.int32)
+    w = np.take_along_axis(p, idx, axis=-1)
+    if renorm:
+        w = w / w.sum(axis=-1, keepdims=True)
+    return idx, w.astype(np.float32)
+
+
+def silu(x: np.ndarray) -> np.ndarray:
+    x = np.asarray(x, dtype=np.float32)
+    return (x / (np.float32(1) + np.exp(-x))).astype(np.float32)
+
+
+def moe_qffn(x_bf16, logits, experts, top_k: int = 2, renorm: bool = True) -> np.ndarray:
+    """Config 3.  experts: list of (wg_p, wg_s, wu_p, wu_s, wd_p, wd_s), int4-g32.
+
+    BUILD CHOICES: gate and up are two separate [F,H] matrices; the intermediate
+    h = silu(x Wg^T) * (x Wu^T) is rounded to bf16 before the down projection
+    (the down GEMM consumes bf16); the weighted sum over the selected experts is
+    accumulated in fp32 and rounded to bf16 once.  Returns bf16 bits [T,H].
+    """
+    idx, w = moe_route(logits, top_k, renorm)
+    t, h_dim = x_bf16.shape
+    y = np.zeros((t, h_dim), dtype=np.float32)
+    for e, (wg_p, wg_s, wu_p, wu_s, wd_p, wd_s) in enumerate(experts):
+        tok, slot = np.nonzero(idx == e)
+        if tok.size == 0:
+            continue
+        xe = x_bf16[tok]
+        g = qgemv_int4g32(xe, wg_p, wg_s)
+        u = qgemv_int4g32(xe, wu_p, wu_s)
+        hmid = f32_to_bf16(silu(g) * u)
+        d = qgemv_int4g32(hmid, wd_p, wd_s)
+        y[tok] += w[tok, slot][:, None] * d
+    return f32_to_bf16(y)
+
+
+# --------------------------------------------------------------------------- quantiser (next-row helper)
+def quantize_int4_g32(w: np.ndarray):
+    """fp32 [N,K] -> (packed uint8 [N,K/2], scale fp16 [N,K/32]); absmax/7 per group, RNE, clamp to [-8,7]."""
+    w = np.asarray(w, dtype=np.float32)
+    n, k = w.shape
+    g = w.reshape(n, k // GROUP, GROUP)
+    s = (np.abs(g).max(axis=2) / np.float32(7)).astype(np.float16)
+    sf = s.astype(np.float32)
+    sf_safe = np.where(sf == 0, np.float32(1), sf)
+    q = np.clip(np.rint(g / sf_safe[:, :, None]), -8, 7).astype(np.int8).reshape(n, k)
+    return pack_int4(q), s
+
+
+def quantize_int8_row(w: np.ndarray):
+    """fp32 [N,K] -> (int8 [N,K], scale fp32 [N]); absmax/127 per row, RNE."""
+    w = np.asarray(w, dtype=np.float32)
+    s = (np.abs(w).max(axis=1) / np.float32(127)).astype(np.float32)
+    s_safe = np.where(s == 0, np.float32(1), s)
+    q = np.clip(np.rint(w / s_safe[:, None]), -127, 127).astype(np.int8)
+    return q, s
+
+
+def rel_l2(a: np.ndarray, ref: np.ndarray) -> float:
+    a = np.asarray(a, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    d = np.linalg.norm(ref)
+    return float(np.linalg.norm(a - ref) / (d if d > 0 else 1.0))
