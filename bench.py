@@ -1,0 +1,240 @@
+#!/usr/bin/env python3
+"""bench.py --gpus 1 --steps K --warmup W  ->  one JSON line.
+
+Workload (N=1): benchmark config 1 at M=1 — the 4-bit group-quantized decode GEMV
+  x bf16 [1,4096] ~N(0,1);  W int4 [14336,4096] packed 2 per byte, group 32 along K, fp16 scale per group
+  ~LogNormal(-5,0.5), zero-point 8;  y fp32 [1,14336].
+A step is one GEMV launch through the C ABI (chadq_gemv_i4g32).  Weights are resident in HBM before the timed
+region.  Steps rotate over 12 distinct copies of the weights (396 MB) so that the 256 MB last-level cache
+cannot serve the stream; the same-buffer ("hot") rate is reported on the side.  Launches are replayed from HIP
+graphs so that Python's per-call cost is not what is measured.
+
+value = algorithmic bytes per launch / average launch duration (HIP events on the launch stream over the
+timed K steps) = the same quantity as roofline.achieved.  Extras: M=4 and M=8, the int8 per-row GEMV
+(config 0) and the prefill dequant-GEMM (config 2, int4 and int8) in TFLOP/s.  cpu_baseline times this build's
+numpy oracle (dequantise to fp32, then sgemv) on the host cores: the reference snapshot has no implementation
+of this path, so there is no reference number to put beside it.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16
+N_COPIES = 12
+SEG = 48                     # launches per captured graph
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=960)
+    ap.add_argument("--warmup", type=int, default=96)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip the side measurements")
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (no collectives are part of it)" % args.gpus,
+              file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from chadslab_amd import QWeightInt4G32, QWeightInt8, _lib, ops
+
+    _lib.load()  # fails loudly if libchadq.so is missing
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    stream = torch.cuda.Stream()
+
+    def bits(t):
+        return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+    def run_steps(fn, steps, warmup):
+        """fn(i) launches step i on the current stream.  Returns (us per step from HIP events, wall us per step)."""
+        with torch.cuda.stream(stream):
+            graphs = {}
+            for length in sorted({min(SEG, steps), steps % SEG} - {0}):
+                for i in range(length):
+                    fn(i)
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    for i in range(length):
+                        fn(i)
+                graphs[length] = g
+            full, rem = divmod(steps, min(SEG, steps))
+            wfull = max(1, warmup // min(SEG, steps))
+            for _ in range(wfull):
+                graphs[min(SEG, steps)].replay()
+            torch.cuda.synchronize()
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            a.record(stream)
+            for _ in range(full):
+                graphs[min(SEG, steps)].replay()
+            if rem:
+                graphs[rem].replay()
+            b.record(stream)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+        return a.elapsed_time(b) * 1000.0 / steps, (t1 - t0) * 1e6 / steps
+
+    # ------------------------------------------------------------------ config 1 (headline)
+    N, K = 14336, 4096
+    rng = np.random.Generator(np.random.PCG64(1001))
+    u = rng.integers(0, 16, (N, K), dtype=np.uint8)
+    packed = (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8)
+    del u
+    scale = rng.lognormal(-5, 0.5, (N, K // 32)).astype(np.float16)
+    x_np = {m: rng.standard_normal((m, K)).astype(np.float32) for m in (1, 4, 8)}
+    base = QWeightInt4G32(torch.from_numpy(packed).to(dev), torch.from_numpy(scale).to(dev))
+    copies = [base] + [QWeightInt4G32(base.packed.clone(), base.scale.clone()) for _ in range(N_COPIES - 1)]
+
+    def gemv_bytes(m):
+        return N * K // 2 + N * (K // 32) * 2 + m * K * 2 + m * N * 4
+
+    results = {}
+    parity = {}
+    for m in (1, 4, 8):
+        if m != 1 and args.no_extras:
+            continue
+        x = torch.from_numpy(x_np[m]).to(torch.bfloat16).to(dev)
+        y = torch.empty(m, N, dtype=torch.float32, device=dev)
+        steps = args.steps if m == 1 else min(args.steps, 480)
+        us, wall = run_steps(lambda i: ops.qgemv(x, copies[i % N_COPIES], out=y), steps, args.warmup)
+        results[m] = (us, wall, steps)
+        if m == 1:
+            from oracle import chadq_oracle as O  # the checker, used once outside the timed region
+
+            parity["gemv_i4g32_m1_rel_l2_vs_f64"] = O.rel_l2(y.cpu().numpy(), O.qgemm_int4g32_f64(bits(x), packed, scale))
+    us1, wall1, steps1 = results[1]
+    achieved = gemv_bytes(1) / us1 * 1e-3  # GB/s
+
+    extras = {}
+    if not args.no_extras:
+        x1 = torch.from_numpy(x_np[1]).to(torch.bfloat16).to(dev)
+        y1 = torch.empty(1, N, dtype=torch.float32, device=dev)
+        us_hot, _ = run_steps(lambda i: ops.qgemv(x1, base, out=y1), 480, 48)
+        extras["gemv_i4g32"] = {
+            "M%d" % m: {"us": round(results[m][0], 3), "GBps": round(gemv_bytes(m) / results[m][0] * 1e-3, 1),
+                        "frac_hbm_peak": round(gemv_bytes(m) / results[m][0] * 1e-3 / HBM_PEAK_GBS, 4)}
+            for m in results
+        }
+        extras["gemv_i4g32"]["M1_same_buffer_every_step"] = {
+            "us": round(us_hot, 3), "GBps": round(gemv_bytes(1) / us_hot * 1e-3, 1),
+            "note": "weights served by the 256 MB last-level cache, not HBM; not a roofline figure"}
+    del copies
+
+    if not args.no_extras:
+        # config 0: int8 per-row GEMV
+        N0, K0 = 16384, 2048
+        r0 = np.random.Generator(np.random.PCG64(1000))
+        x0 = torch.from_numpy(r0.standard_normal((1, K0)).astype(np.float32)).to(dev)
+        w0 = torch.from_numpy(r0.integers(-127, 128, (N0, K0), dtype=np.int8)).to(dev)
+        s0 = torch.from_numpy(r0.uniform(0.001, 0.02, N0).astype(np.float32)).to(dev)
+        c0 = [QWeightInt8(w0.clone(), s0.clone()) for _ in range(N_COPIES)]
+        y0 = torch.empty(1, N0, dtype=torch.float32, device=dev)
+        us0, _ = run_steps(lambda i: ops.qgemv(x0, c0[i % N_COPIES], out=y0), 480, 48)
+        b0 = N0 * K0 + N0 * 4 + K0 * 4 + N0 * 4
+        extras["gemv_i8row_config0"] = {"us": round(us0, 3), "GBps": round(b0 / us0 * 1e-3, 1),
+                                        "frac_hbm_peak": round(b0 / us0 * 1e-3 / HBM_PEAK_GBS, 4)}
+        del c0, w0
+        # config 2: prefill dequant-GEMM, int4 group-32 and int8 per-row
+        M2, N2, K2 = 512, 4096, 4096
+        r2 = np.random.Generator(np.random.PCG64(1002))
+        p2 = torch.from_numpy(r2.integers(0, 256, (N2, K2 // 2), dtype=np.uint8)).to(dev)
+        s2 = torch.from_numpy(r2.lognormal(-5, 0.5, (N2, K2 // 32)).astype(np.float16)).to(dev)
+        x2 = torch.from_numpy(r2.standard_normal((M2, K2)).astype(np.float32)).to(torch.bfloat16).to(dev)
+        y2 = torch.empty(M2, N2, dtype=torch.bfloat16, device=dev)
+        q4 = QWeightInt4G32(p2, s2)
+        q8 = QWeightInt8(torch.from_numpy(r2.integers(-127, 128, (N2, K2), dtype=np.int8)).to(dev),
+                         torch.from_numpy(r2.uniform(0.001, 0.02, N2).astype(np.float32)).to(dev))
+        flop = 2.0 * M2 * N2 * K2
+        for name, qw in (("gemm_i4g32_config2", q4), ("gemm_i8row_config2", q8)):
+            usg, _ = run_steps(lambda i: ops.qgemm(x2, qw, out=y2), 240, 24)
+            extras[name] = {"us": round(usg, 3), "TFLOPs": round(flop / usg * 1e-6, 1),
+                            "frac_bf16_mfma_peak": round(flop / usg * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+
+    # ------------------------------------------------------------------ CPU baseline (rank 0, N=1)
+    cpu = None
+    if not args.no_cpu:
+        from oracle import chadq_oracle as O
+
+        try:
+            from threadpoolctl import threadpool_info
+
+            threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+        except Exception:
+            threads = os.cpu_count() or 1
+        xb = O.f32_to_bf16(x_np[1])
+        t0 = time.perf_counter()
+        O.qgemv_int4g32(xb, packed, scale)
+        first = time.perf_counter() - t0
+        reps = int(min(40, max(3, 15.0 / max(first, 1e-3))))
+        times = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            O.qgemv_int4g32(xb, packed, scale)
+            times.append(time.perf_counter() - t0)
+        med = float(np.median(times))
+        wd = O.dequant_int4g32(packed, scale)
+        xf = O.bf16_to_f32(xb)
+        t2 = []
+        for _ in range(10):
+            t0 = time.perf_counter()
+            xf @ wd.T
+            t2.append(time.perf_counter() - t0)
+        cpu = {
+            "value": round(gemv_bytes(1) / med * 1e-9, 4), "unit": "GB/s", "cores": int(threads), "kind": "port",
+            "sample": "config 1 at M=1, full shape: numpy dequantise-to-fp32 + sgemv, median of %d calls after 1 warm-up "
+                      "(%.1f ms per call); build-written numpy baseline, no reference implementation exists in the snapshot" % (reps, med * 1e3),
+            "predequantised_sgemv_GBps": round(gemv_bytes(1) / float(np.median(t2)) * 1e-9, 3),
+            "host_cpus": os.cpu_count(),
+        }
+
+    out = {
+        "metric": "int4 GEMV HBM GB/s (% peak) + dequant-GEMM TFLOP/s (% MFMA peak), 1 GPU",
+        "value": round(achieved, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": steps1,
+        "warmup": args.warmup,
+        "ms_per_step": round(us1 * 1e-3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 x int4 -> fp32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "config 1: int4 group-32 decode GEMV, M=1, W [14336,4096], x bf16, y fp32",
+                   "M": 1, "N": N, "K": K, "weight_copies_rotated": N_COPIES, "launch": "HIP graph replay, %d launches per graph" % SEG,
+                   "algorithmic_bytes_per_launch": gemv_bytes(1)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "gemv_i4g32_mfma_kernel<1,1>", "wall_clock_us_per_step": round(wall1, 3)},
+        "cpu_baseline": cpu,
+        "parity": parity,
+        "extras": extras,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

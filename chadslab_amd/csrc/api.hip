@@ -1,6 +1,7 @@
 // extern "C" surface of libchadq.so: argument checks, error messages, dispatch.  No allocation, no copies.
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "chadq_common.h"
@@ -43,6 +44,7 @@ int pack_i4_launch(const int8_t *, uint8_t *, int64_t, hipStream_t);
 int dequant_i4g32_launch(const uint8_t *, const uint16_t *, float *, int, int, hipStream_t);
 int dequant_i8row_launch(const int8_t *, const float *, float *, int, int, hipStream_t);
 int gemv_i4g32_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
+int gemv_i4g32_mfma_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
 int gemv_i8row_dispatch(const float *, const int8_t *, const float *, float *, int, int, int, hipStream_t);
 int gemm_i4g32_bf16_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, uint16_t *, int, int, int,
                              hipStream_t);
@@ -110,7 +112,9 @@ int chadq_gemv_i4g32(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *
     if (N == 0) return 0;
     CHADQ_REQUIRE(x_bf16 && wp && scale_f16 && y, CHADQ_ERR_NULL, "chadq_gemv_i4g32: null pointer");
     CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(wp), CHADQ_ERR_ALIGN, "chadq_gemv_i4g32: x and wp must be 16-byte aligned");
-    return gemv_i4g32_dispatch(x_bf16, wp, scale_f16, y, M, N, K, st);
+    static const bool use_dot2 = getenv("CHADQ_GEMV_DOT2") != nullptr;  // development switch
+    if (use_dot2) return gemv_i4g32_dispatch(x_bf16, wp, scale_f16, y, M, N, K, st);
+    return gemv_i4g32_mfma_dispatch(x_bf16, wp, scale_f16, y, M, N, K, st);
 }
 
 int chadq_gemv_i8row(const float *x, const int8_t *w8, const float *scale, float *y, int M, int N, int K,

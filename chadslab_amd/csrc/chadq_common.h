@@ -72,6 +72,29 @@ __device__ __forceinline__ void unpack8_magic(uint32_t w, uint32_t p[4]) {
     p[3] = ((w >> 12) & m) | kBf16Magic;
 }
 
+// (a & mask) | magic in one v_and_or_b32.  The compiler will not form it from C when both constants are
+// literals (a VOP3 instruction cannot carry two), so the constants are passed in registers.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask_reg, uint32_t magic_reg) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(mask_reg), "v"(magic_reg));
+    return r;
+}
+
+// Same as unpack8_magic in 7 instructions: mask_reg = 0x000F000F and magic_reg = kBf16Magic live in VGPRs.
+__device__ __forceinline__ void unpack8_magic_r(uint32_t w, uint32_t mask_reg, uint32_t magic_reg, uint32_t p[4]) {
+    p[0] = and_or(w, mask_reg, magic_reg);
+    p[1] = and_or(w >> 4, mask_reg, magic_reg);
+    p[2] = and_or(w >> 8, mask_reg, magic_reg);
+    p[3] = and_or(w >> 12, mask_reg, magic_reg);
+}
+
+// A constant the optimiser must keep in a vector register.
+__device__ __forceinline__ uint32_t vgpr_const(uint32_t v) {
+    uint32_t r;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(r) : "s"(v));
+    return r;
+}
+
 // Eight consecutive bf16 activations in four registers a[0..3] = (x0,x1),(x2,x3),(x4,x5),(x6,x7) are
 // rearranged to match unpack8_magic's pairing: o[i] = (x_i, x_{i+4}).
 __device__ __forceinline__ void pair_x8(const uint32_t a[4], uint32_t o[4]) {

@@ -27,35 +27,51 @@ __global__ __launch_bounds__(256) void gemv_i4g32_rows_kernel(const uint16_t *__
     if (row0 >= N) return;
     const int KH = K >> 1, G = K >> 5;
 
-    // 1. every weight and scale load of this wave, issued up front
+    // 1. activation loads first.  Memory returns in order, so a wait for the activations must not sit
+    //    behind the weight stream issued next.
+    u32x4 xv[MB][CH][4];
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int k0 = c * 2048 + lane * 32;
+            const u32x4 *xp = reinterpret_cast<const u32x4 *>(x + (size_t)m * K + (k0 < K ? k0 : 0));
+#pragma unroll
+            for (int i = 0; i < 4; ++i) xv[m][c][i] = xp[i];
+        }
+
+    // 2. every weight and scale load of this wave.  Loads are unconditional (a predicated load becomes a
+    //    branch with its own wait and serialises the stream): out-of-range rows and k positions read a
+    //    clamped, valid address and are neutralised through a zero activation / zero scale below.
     u32x4 w[R][CH];
     uint32_t s16[R][CH];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int row = row0 + r;
+        const int row = (row0 + r < N) ? row0 + r : N - 1;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const int k0 = c * 2048 + lane * 32;
-            const bool ok = (row < N) && (k0 < K);
-            w[r][c] = ok ? load_nt_b128(wp + (size_t)row * KH + (k0 >> 1)) : u32x4{0, 0, 0, 0};
-            s16[r][c] = ok ? (uint32_t)__builtin_nontemporal_load(sc + (size_t)row * G + (k0 >> 5)) : 0u;
+            const int kc = (k0 < K) ? k0 : 0;
+            w[r][c] = load_nt_b128(wp + (size_t)row * KH + (kc >> 1));
+            const uint32_t sv = __builtin_nontemporal_load(sc + (size_t)row * G + (kc >> 5));
+            s16[r][c] = (k0 < K) ? sv : 0u;
         }
     }
+    __builtin_amdgcn_sched_barrier(0);  // every load above is issued before anything below may wait
 
-    // 2. activations of this lane's groups, paired to match the unpack order; bias = -136 * sum(x)
+    // activations of this lane's groups, paired to match the unpack order; bias = -136 * sum(x)
     uint32_t xs[MB][CH][16];
     float bias[MB][CH];
 #pragma unroll
     for (int m = 0; m < MB; ++m) {
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
-            const int k0 = c * 2048 + lane * 32;
-            const bool ok = k0 < K;
-            const u32x4 *xp = reinterpret_cast<const u32x4 *>(x + (size_t)m * K + k0);
+            const bool ok = (c * 2048 + lane * 32) < K;
             float sum = 0.f;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                u32x4 v = ok ? xp[i] : u32x4{0, 0, 0, 0};
+                u32x4 v = xv[m][c][i];
+                if (!ok) v = u32x4{0, 0, 0, 0};
                 uint32_t a[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) sum = dot2_bf16(a[j], 0x3F803F80u, sum);  // (1.0, 1.0)
@@ -66,6 +82,7 @@ __global__ __launch_bounds__(256) void gemv_i4g32_rows_kernel(const uint16_t *__
     }
 
     // 3. rows in load order
+    const uint32_t mask_r = vgpr_const(0x000F000Fu), magic_r = vgpr_const(kBf16Magic);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         float acc[MB];
@@ -74,10 +91,10 @@ __global__ __launch_bounds__(256) void gemv_i4g32_rows_kernel(const uint16_t *__
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             uint32_t p[16];
-            unpack8_magic(w[r][c].x, &p[0]);
-            unpack8_magic(w[r][c].y, &p[4]);
-            unpack8_magic(w[r][c].z, &p[8]);
-            unpack8_magic(w[r][c].w, &p[12]);
+            unpack8_magic_r(w[r][c].x, mask_r, magic_r, &p[0]);
+            unpack8_magic_r(w[r][c].y, mask_r, magic_r, &p[4]);
+            unpack8_magic_r(w[r][c].z, mask_r, magic_r, &p[8]);
+            unpack8_magic_r(w[r][c].w, mask_r, magic_r, &p[12]);
             const float s = f16_bits_to_f32((uint16_t)s16[r][c]);
 #pragma unroll
             for (int m = 0; m < MB; ++m) {

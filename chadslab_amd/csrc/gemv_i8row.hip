@@ -21,17 +21,30 @@ __global__ __launch_bounds__(256) void gemv_i8row_rows_kernel(const float *__res
     const int row0 = gw * R;
     if (row0 >= N) return;
 
-    u32x4 w[R][CH];
+    // activation loads first: memory returns in order, so waiting for them must not sit behind the weights
+    f32x4 xv[MB][CH][4];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int row = row0 + r;
+    for (int m = 0; m < MB; ++m)
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const int k0 = c * 1024 + lane * 16;
-            const bool ok = (row < N) && (k0 < K);
-            w[r][c] = ok ? load_nt_b128(w8 + (size_t)row * K + k0) : u32x4{0, 0, 0, 0};
+            const f32x4 *xp = reinterpret_cast<const f32x4 *>(x + (size_t)m * K + ((k0 < K) ? k0 : 0));
+#pragma unroll
+            for (int i = 0; i < 4; ++i) xv[m][c][i] = xp[i];
+        }
+
+    u32x4 w[R][CH];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        // unconditional loads from clamped addresses; out-of-range k meets a zero activation below
+        const int row = (row0 + r < N) ? row0 + r : N - 1;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int k0 = c * 1024 + lane * 16;
+            w[r][c] = load_nt_b128(w8 + (size_t)row * K + ((k0 < K) ? k0 : 0));
         }
     }
+    __builtin_amdgcn_sched_barrier(0);  // every load above is issued before anything below may wait
 
     float xs[MB][CH][16];
     float bias[MB];
@@ -40,12 +53,11 @@ __global__ __launch_bounds__(256) void gemv_i8row_rows_kernel(const float *__res
         float sum = 0.f;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
-            const int k0 = c * 1024 + lane * 16;
-            const bool ok = k0 < K;
-            const f32x4 *xp = reinterpret_cast<const f32x4 *>(x + (size_t)m * K + k0);
+            const bool ok = (c * 1024 + lane * 16) < K;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const f32x4 v = ok ? xp[i] : f32x4{0.f, 0.f, 0.f, 0.f};
+                f32x4 v = xv[m][c][i];
+                if (!ok) v = f32x4{0.f, 0.f, 0.f, 0.f};
                 xs[m][c][4 * i + 0] = v.x;
                 xs[m][c][4 * i + 1] = v.y;
                 xs[m][c][4 * i + 2] = v.z;

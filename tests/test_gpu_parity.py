@@ -1,0 +1,262 @@
+"""GPU parity: the HIP path, called through the C ABI (chadslab_amd.ops -> ctypes -> libchadq.so), against the
+CPU oracle on the same seeded inputs.  Bit-exact for unpack/pack/dequant and integer accumulation; rel-L2
+<= 1e-3 for fp32 outputs and <= 1e-2 for bf16 outputs against the float64 ground truth (tolerances from the
+benchmark statement).  Full benchmark shapes are covered too: the numpy oracle finishes them in seconds.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import chadq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL_F32 = 1e-3   # fp32 out
+TOL_BF16 = 1e-2  # bf16 out
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from chadslab_amd import _lib, ops as _ops
+
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    _lib.load()  # raises if libchadq.so is missing: there is no fallback to hide behind
+    return _ops
+
+
+def rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+def bits(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def bf16_tensor(b):
+    return torch.from_numpy(b.view(np.int16)).view(torch.bfloat16).to(DEV)
+
+
+def i4_case(seed, m, n, k, integer_x=False):
+    from chadslab_amd import QWeightInt4G32
+
+    r = rng(seed)
+    u = r.integers(0, 16, (n, k), dtype=np.uint8)
+    packed = (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8)
+    s = r.lognormal(-5, 0.5, (n, k // 32)).astype(np.float16)
+    x = r.integers(-8, 9, (m, k)).astype(np.float32) if integer_x else r.standard_normal((m, k)).astype(np.float32)
+    xb = O.f32_to_bf16(x)
+    qw = QWeightInt4G32(torch.from_numpy(packed).to(DEV), torch.from_numpy(s).to(DEV))
+    return packed, s, xb, qw
+
+
+def i8_case(seed, m, n, k):
+    from chadslab_amd import QWeightInt8
+
+    r = rng(seed)
+    x = r.standard_normal((m, k)).astype(np.float32)
+    w = r.integers(-127, 128, (n, k), dtype=np.int8)
+    s = r.uniform(0.001, 0.02, n).astype(np.float32)
+    return x, w, s, QWeightInt8(torch.from_numpy(w).to(DEV), torch.from_numpy(s).to(DEV))
+
+
+# ------------------------------------------------------------------ unpack / pack / dequant: bit-exact
+@pytest.mark.parametrize("nbytes", [0, 1, 15, 16, 17, 255, 256, 4096 + 7, 1 << 20])
+def test_unpack_bit_exact(ops, nbytes):
+    wp = rng(nbytes).integers(0, 256, nbytes, dtype=np.uint8)
+    if nbytes >= 256:
+        wp[:256] = np.arange(256)  # every byte value
+    out = ops.unpack_int4(torch.from_numpy(wp).to(DEV)).cpu().numpy()
+    assert np.array_equal(out, O.unpack_int4(wp[None])[0] if nbytes else np.zeros(0, np.int8))
+
+
+def test_unpack_unaligned_view(ops):
+    wp = rng(3).integers(0, 256, 1001, dtype=np.uint8)
+    t = torch.from_numpy(wp).to(DEV)[1:]  # data pointer off 16-byte alignment
+    assert np.array_equal(ops.unpack_int4(t).cpu().numpy(), O.unpack_int4(wp[None, 1:])[0])
+
+
+def test_pack_roundtrip(ops):
+    q = rng(4).integers(-8, 8, (33, 130), dtype=np.int8)
+    p = ops.pack_int4(torch.from_numpy(q).to(DEV))
+    assert np.array_equal(p.cpu().numpy(), O.pack_int4(q))
+    assert np.array_equal(ops.unpack_int4(p).cpu().numpy(), q)
+
+
+def test_dequant_exact(ops):
+    packed, s, _, qw = i4_case(5, 1, 96, 256)
+    assert np.array_equal(ops.dequantize(qw).cpu().numpy(), O.dequant_int4g32(packed, s))
+    _, w, s8, q8 = i8_case(6, 1, 50, 70)
+    assert np.array_equal(ops.dequantize(q8).cpu().numpy(), O.dequant_int8(w, s8))
+
+
+# ------------------------------------------------------------------ golden fixtures
+def test_golden_int4(ops):
+    from chadslab_amd import QWeightInt4G32
+
+    g = np.load(os.path.join(GOLD, "i4g32_n64_k128.npz"))
+    qw = QWeightInt4G32(torch.from_numpy(g["packed"]).to(DEV), torch.from_numpy(g["scale"]).to(DEV))
+    x = bf16_tensor(g["x_bf16"])
+    assert np.array_equal(ops.unpack_int4(qw.packed).cpu().numpy(), g["q"])
+    assert np.array_equal(ops.dequantize(qw).cpu().numpy(), g["dequant"])
+    assert O.rel_l2(ops.qgemv(x, qw).cpu().numpy(), g["y_f64"]) <= TOL_F32
+    assert O.rel_l2(O.bf16_to_f32(bits(ops.qgemm(x, qw))), g["y_f64"]) <= TOL_BF16
+
+
+def test_golden_int8(ops):
+    from chadslab_amd import QWeightInt8
+
+    g = np.load(os.path.join(GOLD, "i8row_n64_k128.npz"))
+    q8 = QWeightInt8(torch.from_numpy(g["w"]).to(DEV), torch.from_numpy(g["scale"]).to(DEV))
+    assert O.rel_l2(ops.qgemv(torch.from_numpy(g["x_f32"]).to(DEV), q8).cpu().numpy(), g["y_f64"]) <= TOL_F32
+    assert O.rel_l2(O.bf16_to_f32(bits(ops.qgemm(bf16_tensor(g["x_bf16"]), q8))), g["yb_f64"]) <= TOL_BF16
+
+
+# ------------------------------------------------------------------ GEMV int4 (config 1)
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8, 16])
+@pytest.mark.parametrize("n,k", [(64, 128), (33, 32), (100, 4160), (48, 12288), (257, 2048), (1000, 4096), (16, 8192)])
+def test_gemv_int4_shapes(ops, m, n, k):
+    packed, s, xb, qw = i4_case(100 + m + n + k, m, n, k)
+    y = ops.qgemv(bf16_tensor(xb), qw).cpu().numpy()
+    assert y.shape == (m, n) and np.isfinite(y).all()
+    assert O.rel_l2(y, O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_F32
+
+
+@pytest.mark.parametrize("m", [1, 4, 8])
+def test_gemv_int4_config1_full_size(ops, m):
+    packed, s, xb, qw = i4_case(1001, m, 14336, 4096)
+    y = ops.qgemv(bf16_tensor(xb), qw).cpu().numpy()
+    assert O.rel_l2(y, O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_F32
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 14336, 4096), (8, 512, 4096), (4, 96, 256), (2, 40, 96)])
+def test_gemv_int4_integer_accumulation_bit_exact(ops, m, n, k):
+    from chadslab_amd import QWeightInt4G32
+
+    packed, _, xb, qw = i4_case(7, m, n, k, integer_x=True)
+    ones = QWeightInt4G32(qw.packed, torch.ones_like(qw.scale))
+    y = ops.qgemv(bf16_tensor(xb), ones).cpu().numpy()
+    brute = O.bf16_to_f32(xb).astype(np.int64) @ O.unpack_int4(packed).astype(np.int64).T
+    assert np.abs(brute).max() < 2 ** 24
+    assert np.array_equal(y.astype(np.int64), brute) and np.array_equal(y, brute.astype(np.float32))
+
+
+def test_gemv_int4_row_consistency_and_linearity(ops):
+    packed, s, xb, qw = i4_case(8, 8, 512, 4096)
+    x = bf16_tensor(xb)
+    y8 = ops.qgemv(x, qw).cpu().numpy()
+    for r in (0, 3, 7):
+        y1 = ops.qgemv(x[r:r + 1].contiguous(), qw).cpu().numpy()
+        assert O.rel_l2(y1[0], y8[r]) <= 1e-6  # same products, possibly another summation order
+    a = rng(9).integers(-64, 64, (1, 4096)).astype(np.float32)
+    b = rng(10).integers(-64, 64, (1, 4096)).astype(np.float32)
+    ya, yb, yab = (ops.qgemv(bf16_tensor(O.f32_to_bf16(v)), qw).cpu().numpy() for v in (a, b, a + b))
+    assert O.rel_l2(yab, ya + yb) <= 1e-5
+
+
+def test_gemv_int4_zero_weights_and_special_scales(ops):
+    from chadslab_amd import QWeightInt4G32
+
+    n, k = 64, 4096
+    x = bf16_tensor(O.f32_to_bf16(rng(11).standard_normal((2, k)).astype(np.float32)))
+    zero = QWeightInt4G32(torch.full((n, k // 2), 0x88, dtype=torch.uint8, device=DEV), torch.ones(n, k // 32, dtype=torch.float16, device=DEV))
+    y = ops.qgemv(x, zero).cpu().numpy()
+    # u = 8 everywhere: the 128+u offset must cancel; what is left is fp32 rounding of sums near 136*sum|x|,
+    # about 1e-4 of the size a typical output has for these shapes (~300)
+    assert np.abs(y).max() <= 2e-2
+    # one-hot activation returns one dequantised column exactly
+    packed, s, _, qw = i4_case(12, 1, n, k)
+    d = O.dequant_int4g32(packed, s)
+    for kk in (0, 31, 32, 2047, 4095):
+        e = np.zeros((1, k), np.float32)
+        e[0, kk] = 1.0
+        assert np.array_equal(ops.qgemv(bf16_tensor(O.f32_to_bf16(e)), qw).cpu().numpy()[0], d[:, kk])
+
+
+# ------------------------------------------------------------------ GEMV int8 (config 0)
+@pytest.mark.parametrize("m,n,k", [(1, 16384, 2048), (1, 64, 16), (3, 100, 1040), (2, 77, 4096), (16, 40, 256)])
+def test_gemv_int8(ops, m, n, k):
+    x, w, s, q8 = i8_case(1000 if (n, k) == (16384, 2048) else 20 + n, m, n, k)
+    y = ops.qgemv(torch.from_numpy(x).to(DEV), q8).cpu().numpy()
+    assert O.rel_l2(y, O.qgemv_int8_f64(x, w, s)) <= TOL_F32
+
+
+def test_gemv_int8_integer_exact(ops):
+    from chadslab_amd import QWeightInt8
+
+    r = rng(21)
+    x = r.integers(-8, 9, (2, 2048)).astype(np.float32)
+    w = r.integers(-127, 128, (300, 2048), dtype=np.int8)
+    q8 = QWeightInt8(torch.from_numpy(w).to(DEV), torch.ones(300, device=DEV))
+    y = ops.qgemv(torch.from_numpy(x).to(DEV), q8).cpu().numpy()
+    assert np.array_equal(y.astype(np.int64), x.astype(np.int64) @ w.astype(np.int64).T)
+
+
+# ------------------------------------------------------------------ prefill GEMM (config 2)
+@pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (1, 64, 128), (37, 100, 96), (130, 70, 288), (5, 33, 32), (128, 64, 256), (200, 192, 1056)])
+def test_gemm_int4(ops, m, n, k):
+    packed, s, xb, qw = i4_case(1002 if m == 512 else 30 + m, m, n, k)
+    y = O.bf16_to_f32(bits(ops.qgemm(bf16_tensor(xb), qw)))
+    assert y.shape == (m, n)
+    assert O.rel_l2(y, O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_BF16
+
+
+@pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (3, 40, 16), (129, 65, 272), (64, 128, 128)])
+def test_gemm_int8(ops, m, n, k):
+    x, w, s, q8 = i8_case(40 + m, m, n, k)
+    xb = O.f32_to_bf16(x)
+    y = O.bf16_to_f32(bits(ops.qgemm(bf16_tensor(xb), q8)))
+    assert O.rel_l2(y, O.qgemm_int8_f64(xb, w, s)) <= TOL_BF16
+
+
+def test_gemm_agrees_with_gemv_at_m8(ops):
+    packed, s, xb, qw = i4_case(50, 8, 1024, 4096)
+    x = bf16_tensor(xb)
+    gemv = ops.qgemv(x, qw).cpu().numpy()
+    gemm = O.bf16_to_f32(bits(ops.qgemm(x, qw)))
+    assert O.rel_l2(gemm, gemv) <= TOL_BF16
+
+
+def test_gemm_int4_integer_exact_when_scales_are_one(ops):
+    from chadslab_amd import QWeightInt4G32
+
+    packed, _, xb, qw = i4_case(51, 64, 128, 512, integer_x=True)
+    ones = QWeightInt4G32(qw.packed, torch.ones_like(qw.scale))
+    # |sum| <= 512*8*8 = 32768 needs 16 bits: bf16 output cannot hold it, so compare after rounding the
+    # exact integer result to bf16 (fp32 accumulation of exact integers is exact)
+    brute = (O.bf16_to_f32(xb).astype(np.int64) @ O.unpack_int4(packed).astype(np.int64).T).astype(np.float32)
+    assert np.array_equal(bits(ops.qgemm(bf16_tensor(xb), ones)), O.f32_to_bf16(brute))
+
+
+# ------------------------------------------------------------------ operator layer and error behaviour
+def test_qlinear_dispatch(ops):
+    packed, s, xb, qw = i4_case(60, 6, 128, 256)
+    x = bf16_tensor(xb).reshape(2, 3, 256)
+    y = ops.qlinear(x, qw)
+    assert y.shape == (2, 3, 128) and y.dtype == torch.float32  # decode sizes come back in fp32
+    assert O.rel_l2(y.reshape(6, 128).cpu().numpy(), O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_F32
+    packed, s, xb, qw = i4_case(61, 40, 128, 256)
+    y = ops.qlinear(bf16_tensor(xb), qw)
+    assert y.dtype == torch.bfloat16 and O.rel_l2(O.bf16_to_f32(bits(y)), O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_BF16
+    assert ops.qlinear(bf16_tensor(xb), qw, out_dtype=torch.float32).dtype == torch.float32
+
+
+def test_errors_surface_as_exceptions(ops):
+    from chadslab_amd import QWeightInt4G32, _lib
+
+    _, _, xb, qw = i4_case(62, 1, 64, 128)
+    with pytest.raises(ValueError):
+        ops.qgemv(bf16_tensor(xb)[:, :96].contiguous(), qw)          # K mismatch
+    with pytest.raises(ValueError):
+        ops.qgemv(bf16_tensor(xb).float(), qw)                       # wrong dtype
+    with pytest.raises(ValueError):
+        ops.qgemv(bf16_tensor(np.zeros((17, 128), np.uint16)), qw)   # M beyond the GEMV's range
+    lib = _lib.load()
+    assert lib.chadq_gemv_i4g32(None, None, None, None, 1, 64, 128, None) == -1
+    assert b"null" in lib.chadq_last_error()
+    assert lib.chadq_gemv_i4g32(None, None, None, None, 1, 64, 100, None) == -2
+    assert b"multiple of 32" in lib.chadq_last_error()
+    assert lib.chadq_gemv_i4g32(None, None, None, None, 1, 0, 128, None) == 0  # empty output: nothing to do
