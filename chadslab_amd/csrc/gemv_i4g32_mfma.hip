@@ -1,146 +1,171 @@
-// Decode GEMV on int4 group-32 weights, matrix-core form, for 1 <= M <= 8 activation rows.
+// Decode GEMV on int4 group-32 weights, matrix-core form, for 1 <= M <= 8 activation rows per launch.
 //
 // The kernel is HBM-bound by design; the matrix core is used only because it makes the dot products free
 // of vector-ALU work, which is what limits a plain dot-product kernel on this shape (about 12 VALU
-// instructions per 8 nibbles are affordable at full HBM rate; unpack alone costs 7).
+// instructions per 8 nibbles are affordable at full HBM rate; unpacking alone costs 7).
 //
 // One v_mfma_f32_16x16x32_bf16 step, D[16x16] += A[16x32] * B[32x16]:
-//   B = weights.  Lane (n = lane%16, j = lane/16) loads 16 packed bytes of output row n0+n: the 32 nibbles
-//       of scale group 4c+j.  A wave-wide load is 16 rows x 64 contiguous bytes.  The four 32-bit words of
-//       the load are the B operands of four MFMA steps t = 0..3 (8 k each); lane group j supplies k-slots
-//       8j..8j+7.  Nibbles become bf16 128+u by OR-ing into 0x4300 (exact).
-//   A = activations, block diagonal.  Row i = 4j'+m of A is activation row m restricted to lane group j':
-//       A[4j'+m][k-slot group j] = x[m][those 8 k] if j == j', else 0.  So D[4j+m][n] is the dot product of
-//       activation row m with ONE scale group (4c+j) of weight row n, and the lane that holds D[4j..4j+3][n]
-//       is lane (n, j) - the lane that loaded that group and its scale.  One fp32 FMA per activation row
-//       applies the scale; nothing crosses lanes inside the K loop.
+//   B = weights.  The 16 columns are P = 16/HP weight rows times HP "K-parts": column n = h*P + r.  Lane
+//       (n, j = lane/16) loads 16 packed bytes of row r: the 32 nibbles of scale group (c*HP + h)*4 + j at
+//       step c.  A wave-wide load therefore covers P rows x (HP * 64) contiguous bytes: 4 rows x 256 B for
+//       HP = 4, 16 rows x 64 B for HP = 1.  The four 32-bit words of the load are the B operands of four
+//       MFMA steps t = 0..3 (8 k each); lane group j supplies k-slots 8j..8j+7.  Nibbles become bf16 128+u
+//       by OR-ing them into 0x4300 (exact).
+//   A = activations, block diagonal.  Row i = 4j' + v, v = h'*MPASS + m (MPASS = 4/HP activation rows per
+//       pass): A[i][k-slots of lane group j] = x[m][the 8 k of group (c*HP + h')*4 + j', word t] if j == j',
+//       else 0.  D[4j + v][n] is then the dot product of activation row m with ONE scale group of weight
+//       row r - meaningful where the column's K-part h equals h' - and the lane that holds D[4j..4j+3][n]
+//       is lane (n, j), the lane that loaded exactly that group and owns its scale.  One fp32 FMA per D
+//       register applies the scale; nothing crosses lanes inside the K loop.  Entries with h' != h are
+//       computed and never used.
 //   C = -136 * sum of the group's activations, which turns 128+u into u-8.  For integer-valued activations
 //       every term is an exact fp32 integer, so integer accumulation stays bit-exact.
-// Up to 4 activation rows ride in one pass; MP = 2 runs two passes over the same unpacked weights.
+// HP trades activation rows per pass for contiguity of the weight stream: M = 1 runs HP = 4, M = 2 runs
+// HP = 2, M >= 3 runs HP = 1 (two passes over the same unpacked weights for M > 4).
 //
-// Workgroup = RBW row blocks (16 rows each) x 4 K-slices, one wave each.  K is consumed in chunks of 4096
-// (1024 k = 8 steps per wave).  Every wave issues, in this order, its activation loads, ONE load for its
-// 16 x 32 tile of scales (parked in a wave-private LDS tile and read back 2 bytes at a time) and its eight
-// weight loads, all before the first wait; memory returns in order, so what is needed first is asked for
-// first.  The workgroup then stages the chunk's activations into LDS in A-operand order while the weights
-// are still in flight.  Partial
-// sums of the 4 lane groups and 4 K-slices meet in LDS at the end; results are written once, in a fixed
-// order (deterministic).
+// Workgroup = 4*RBW waves; each group of 4 waves covers 16 weight rows.  K is consumed in chunks of 4096;
+// a wave takes 8 steps of a chunk (8 x 16 B per lane in flight), so 4/HP waves split a chunk of one row
+// block.  Every wave issues, in this order, its activation loads, ONE load for its tile of scales (parked
+// in a wave-private LDS tile and read back 2 bytes at a time) and its first D weight loads, all before the
+// first wait: memory returns in order, so what is needed first is asked for first.  Step i issues weight
+// load i+D when its own data has arrived (prefetch distance D): a wave's requests are then spread over the
+// whole stream and its last bytes meet one step of arithmetic instead of eight.  The workgroup stages the
+// chunk's activations into LDS in A-operand order while the weights are still in flight.  Partial sums
+// of lane groups, K-parts and K-slices meet in LDS at the end; results are written once, in a fixed order
+// (deterministic).
 #include "chadq_common.h"
 
 namespace chadq {
 
-constexpr int KC = 4096;             // k per chunk
-constexpr int CSC = KC / 128;        // 128-k steps per chunk (32)
-constexpr int XA_BYTES = CSC * 1024; // A operands of one pass for one chunk: [c][t][j][m] x 16 B
-constexpr int NX_BYTES = (KC / 32) * 16;  // C operands: [group][m] fp32
+constexpr int KC = 4096;  // k per chunk
 constexpr int ZERO_BYTES = 1024;
 
-template <int MP, int RBW>
-struct GemvLds {
+template <int MT, int HP, int S, int RBW>
+struct GemvCfg {
+    static constexpr int P = 16 / HP;                    // weight rows per MFMA tile
+    static constexpr int MPASS = 4 / HP;                 // activation rows per pass
+    static constexpr int MP = (MT + MPASS - 1) / MPASS;  // passes
+    static constexpr int STEPS = KC / (128 * HP);        // steps per chunk of one row block
+    static constexpr int KS = STEPS / S;                 // waves that split a chunk of one row block (S steps each)
+    static constexpr int UR = P * 4 / KS;                // weight rows covered by a group of 4 waves
+    static_assert(KS >= 1 && KS <= 4 && KS * S == STEPS, "a chunk of one row block is split over 1, 2 or 4 waves");
+    static constexpr int XA_BYTES = STEPS * 1024;        // A operands of one pass: [c][t][j][v] x 16 B
+    static constexpr int NX_BYTES = STEPS * 64;          // C operands of one pass: [c][j][v] fp32
     static constexpr int PASS = XA_BYTES + NX_BYTES;
     static constexpr int ZERO_OFF = MP * PASS;
-    static constexpr int SC_OFF = ZERO_OFF + ZERO_BYTES;  // per-wave scale tiles: 16 rows x (64 B + 16 pad)
-    static constexpr int SC_WAVE = 16 * 80;
+    static constexpr int SC_OFF = ZERO_OFF + ZERO_BYTES;
+    static constexpr int SC_PPR = S * HP / 2;            // 16-byte pieces (8 groups) per scale tile row
+    static constexpr int SC_PITCH = SC_PPR * 16 + 16;    // scale tile row: S*4*HP fp16 + pad
+    static constexpr int SC_WAVE = P * SC_PITCH;
     static constexpr int OPER_BYTES = SC_OFF + RBW * 4 * SC_WAVE;
     static constexpr int RED_BYTES = RBW * 4 * 64 * MP * 16;  // reuses the operand area after the K loop
     static constexpr int TOTAL = OPER_BYTES > RED_BYTES ? OPER_BYTES : RED_BYTES;
+    static constexpr int T = 256 * RBW;
+    static constexpr int XI = (MPASS * (KC / 8) + T - 1) / T;  // 16-byte activation pieces per thread per pass
 };
 
-// waves_per_eu(4): at most 128 VGPRs, which also makes the compiler pick the MFMA form that writes VGPRs
-// MT = number of activation rows (compile time, so that no staging load hides behind a branch).
-template <int MT, int RBW>
-__global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) void gemv_i4g32_mfma_kernel(const uint16_t *__restrict__ x,
-                                                                    const uint8_t *__restrict__ wp,
-                                                                    const uint16_t *__restrict__ sc,
-                                                                    float *__restrict__ y, int N, int K) {
-    constexpr int M = MT, MP = (MT + 3) / 4;
-    typedef GemvLds<MP, RBW> L;
-    constexpr int T = 256 * RBW;
+// waves_per_eu(4): at most 128 VGPRs, which also makes the compiler pick the MFMA form that writes VGPRs.
+template <int MT, int HP, int S, int RBW, int D>
+__global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) void gemv_i4g32_mfma_kernel(
+    const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
+    float *__restrict__ y, int N, int K) {
+    typedef GemvCfg<MT, HP, S, RBW> C;
+    constexpr int M = MT, MP = C::MP, MPASS = C::MPASS, P = C::P, KS = C::KS, T = C::T, XI = C::XI;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int rbl = wave >> 2, ks = wave & 3;
+    const int unit = wave >> 2, wv = wave & 3;     // group of 4 waves (UR rows) inside the workgroup, wave inside it
+    const int rbs = wv / KS, ks = wv % KS;         // row block inside the unit, K-slice
     const int nl = lane & 15, j = lane >> 4;
-    const int n0 = (blockIdx.x * RBW + rbl) * 16;
+    const int h = nl / P, r = nl % P;              // K-part and row of this lane's MFMA column
+    const int n0 = (blockIdx.x * RBW + unit) * C::UR + rbs * P;
     const int KH = K >> 1, G = K >> 5;
-    const int row = (n0 + nl < N) ? n0 + nl : N - 1;
+    const int row = (n0 + r < N) ? n0 + r : N - 1;
     const uint32_t wrow = (uint32_t)row * (uint32_t)KH;  // byte offset; the host checks N*K/2 < 2^31
-    const uint32_t srow = (uint32_t)row * (uint32_t)G;
     const uint32_t mask_r = vgpr_const(0x000F000Fu), magic_r = vgpr_const(kBf16Magic);
 
     // the zero block that A lanes off the diagonal (and padding activation rows) read from
-    for (int o = tid * 16; o < ZERO_BYTES; o += T * 16) *reinterpret_cast<u32x4 *>(lds + L::ZERO_OFF + o) = u32x4{0, 0, 0, 0};
+    for (int o = tid * 16; o < ZERO_BYTES; o += T * 16)
+        *reinterpret_cast<u32x4 *>(lds + C::ZERO_OFF + o) = u32x4{0, 0, 0, 0};
 
-    // A-operand address of this lane per pass: real data only where row 4j'+m meets k-slot group j'=j and
-    // activation row 4p+m exists; every other lane reads zeros (stride 0 keeps it inside the zero block)
+    // A-operand address of this lane per pass: real data only on the diagonal (row 4j'+v meets k-slot
+    // group j = j') and where activation row p*MPASS + v%MPASS exists; all other lanes read zeros (stride
+    // 0 keeps them inside the zero block)
     uint32_t a_base[MP], a_step[MP];
 #pragma unroll
     for (int p = 0; p < MP; ++p) {
-        const bool act = (((lane & 15) >> 2) == j) && (4 * p + (lane & 3) < M);
-        a_base[p] = act ? (uint32_t)(p * L::PASS + ks * 8192 + 64 * j + 16 * (lane & 3)) : (uint32_t)L::ZERO_OFF;
-        a_step[p] = act ? 1024u : 0u;  // LDS bytes between this wave's consecutive 128-k steps
+        const int v = lane & 3;
+        const bool act = (((lane & 15) >> 2) == j) && (p * MPASS + (v % MPASS) < M);
+        a_base[p] = act ? (uint32_t)(p * C::PASS + ks * S * 1024 + 64 * j + 16 * v) : (uint32_t)C::ZERO_OFF;
+        a_step[p] = act ? 1024u : 0u;
     }
 
     f32x4 acc[MP];
 #pragma unroll
     for (int p = 0; p < MP; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    constexpr int XI = (4 * (KC / 8)) / T;  // activation pieces (16 B) per thread per pass when 4 rows are live
+    // scale tile of this wave: P rows x 32*HP groups; lane -> (row, 8-group piece) for the single load
+    uint8_t *sct = lds + C::SC_OFF + wave * C::SC_WAVE;
+    const int srow_l = lane / C::SC_PPR, spiece = lane % C::SC_PPR;  // lanes beyond P rows repeat the last row
+    const int srow = (n0 + srow_l < N) ? n0 + srow_l : N - 1;
+
     for (int kc0 = 0; kc0 < K; kc0 += KC) {
-        // 1. activation loads FIRST: memory returns in order, so the wait for these must not sit behind the
-        //    weight stream.  Piece `it` = tid + T*r of pass p: row m = it / 512, i8 = it % 512 = 16c + 4j + t.
+        // 1. activation loads FIRST.  Piece `it` = tid + T*q of pass p: row m = it / 512, i8 = it % 512.
         u32x4 xr[MP][XI];
 #pragma unroll
         for (int p = 0; p < MP; ++p)
 #pragma unroll
-            for (int r = 0; r < XI; ++r) {
-                const int m = (T * r) / (KC / 8);  // same for the whole workgroup: T divides KC/8
-                if (4 * p + m >= M) continue;      // compile-time after unrolling
-                const int k = kc0 + 8 * ((tid + T * r) % (KC / 8));
-                xr[p][r] = *reinterpret_cast<const u32x4 *>(x + (k < K ? (size_t)(4 * p + m) * K + k : 0));
+            for (int q = 0; q < XI; ++q) {
+                const int m = (T * q) / (KC / 8);  // same for the whole workgroup: T divides KC/8
+                if (m >= MPASS || p * MPASS + m >= M) continue;  // compile time after unrolling
+                const int k = kc0 + 8 * ((tid + T * q) % (KC / 8));
+                xr[p][q] = *reinterpret_cast<const u32x4 *>(x + (k < K ? (size_t)(p * MPASS + m) * K + k : 0));
             }
 
-        // 2. the wave's scale tile: 16 rows x 32 groups (64 B per row) in one load; lane (n,j) takes groups
-        //    8j..8j+7 of the wave's K-slice.  Needs G % 8 == 0 (16-byte aligned rows), checked on the host.
-        const int gs = (kc0 >> 5) + 32 * ks + 8 * j;
-        u32x4 sv = *reinterpret_cast<const u32x4 *>(sc + (srow + (uint32_t)(gs < G ? gs : 0)));
+        // 2. the wave's scale tile in one load.  Needs G % 8 == 0 (16-byte aligned pieces), checked on the host.
+        const int gs = (kc0 >> 5) + ks * S * 4 * HP + spiece * 8;
+        u32x4 sv = *reinterpret_cast<const u32x4 *>(sc + ((size_t)srow * G + (gs < G ? gs : 0)));
         if (gs >= G) sv = u32x4{0, 0, 0, 0};
 
-        // 3. this wave's weight loads for the chunk: steps c = 8*ks + i, lane (n,j) takes group 4c+j
-        u32x4 w[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int g = (kc0 >> 5) + 4 * (8 * ks + i) + j;
+        // 3. the wave's weight loads for the chunk: steps c = 8*ks + i, lane takes group (c*HP + h)*4 + j
+        //    Only the first D are issued now; step i issues load i+D once its own data has arrived, so a
+        //    wave's requests are spread over the stream and its last data meets one step of work, not S.
+        u32x4 w[S];
+        auto issue_w = [&](int i) {
+            const int g = (kc0 >> 5) + ((S * ks + i) * HP + h) * 4 + j;
             w[i] = load_nt_b128(wp + (wrow + (uint32_t)(g < G ? g : 0) * 16u));
-        }
+        };
+#pragma unroll
+        for (int i = 0; i < (D < S ? D : S); ++i) issue_w(i);
         __builtin_amdgcn_sched_barrier(0);  // every load above is issued before anything below may wait
 
-        // 4. stage the activations: 16-byte pieces (8 k) -> [c][t][j][m], paired for the unpack order, and
+        // 4. stage the activations: 16-byte pieces (8 k) -> [c][t][j][v], paired for the unpack order, and
         //    the C operands -136 * (sum of the group's 32 activations)
         __syncthreads();  // previous chunk's operand reads (or the zero fill) are done
-        uint8_t *sct = lds + L::SC_OFF + wave * L::SC_WAVE;  // wave-private: no barrier between write and reads
-        *reinterpret_cast<u32x4 *>(sct + nl * 80 + j * 16) = sv;
+        if (srow_l < P) *reinterpret_cast<u32x4 *>(sct + srow_l * C::SC_PITCH + spiece * 16) = sv;  // wave-private tile
 #pragma unroll
         for (int p = 0; p < MP; ++p)
 #pragma unroll
-            for (int r = 0; r < XI; ++r) {
-                const int m = (T * r) / (KC / 8);  // same for the whole workgroup: T divides KC/8
-                if (4 * p + m >= M) continue;      // padding row (compile time): its A lanes read the zero block
-                const int i8 = (tid + T * r) % (KC / 8);
-                u32x4 v = xr[p][r];
+            for (int q = 0; q < XI; ++q) {
+                const int m = (T * q) / (KC / 8);
+                if (m >= MPASS || p * MPASS + m >= M) continue;  // padding row: its A lanes read the zero block
+                const int i8 = (tid + T * q) % (KC / 8);
+                u32x4 v = xr[p][q];
                 if (kc0 + 8 * i8 >= K) v = u32x4{0, 0, 0, 0};
                 uint32_t a[4] = {v.x, v.y, v.z, v.w}, o[4];
                 float sum = 0.f;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) sum = dot2_bf16(a[q], 0x3F803F80u, sum);
+                for (int e = 0; e < 4; ++e) sum = dot2_bf16(a[e], 0x3F803F80u, sum);
                 pair_x8(a, o);
-                const int c = i8 >> 4, jj = (i8 >> 2) & 3, t = i8 & 3;
-                *reinterpret_cast<u32x4 *>(lds + p * L::PASS + c * 1024 + t * 256 + jj * 64 + m * 16) =
+                // chunk-local group gl = (c*HP + h')*4 + j'
+                const int gl = i8 >> 2, t = i8 & 3;
+                const int c = gl / (4 * HP), hh = (gl >> 2) % HP, jj = gl & 3;
+                const int vv = hh * MPASS + m;
+                *reinterpret_cast<u32x4 *>(lds + p * C::PASS + c * 1024 + t * 256 + jj * 64 + vv * 16) =
                     u32x4{o[0], o[1], o[2], o[3]};
                 sum += dpp_f32<0xB1, 0xF>(sum);  // the 4 pieces of a group sit in 4 adjacent lanes
                 sum += dpp_f32<0x4E, 0xF>(sum);
                 if (t == 0)
-                    *reinterpret_cast<float *>(lds + p * L::PASS + XA_BYTES + (i8 >> 2) * 16 + m * 4) = -kMagicBias * sum;
+                    *reinterpret_cast<float *>(lds + p * C::PASS + C::XA_BYTES + (c * 4 + jj) * 16 + vv * 4) = -kMagicBias * sum;
             }
         __syncthreads();
 
@@ -149,17 +174,24 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
 #pragma unroll
         for (int p = 0; p < MP; ++p) a_addr[p] = a_base[p];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int c = 8 * ks + i;
+        for (int i = 0; i < S; ++i) {
+            const int c = S * ks + i;
             uint32_t pw[16];
+            if (D < S) {
+                // wait for this step's weights, then put the next request in the queue before computing
+                asm volatile("" : "+v"(w[i]));
+                if (i + D < S) issue_w(i + D);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             unpack8_magic_r(w[i].x, mask_r, magic_r, &pw[0]);
             unpack8_magic_r(w[i].y, mask_r, magic_r, &pw[4]);
             unpack8_magic_r(w[i].z, mask_r, magic_r, &pw[8]);
             unpack8_magic_r(w[i].w, mask_r, magic_r, &pw[12]);
-            const float s = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(sct + nl * 80 + (4 * i + j) * 2));
+            const float s = f16_bits_to_f32(
+                *reinterpret_cast<const uint16_t *>(sct + r * C::SC_PITCH + ((i * HP + h) * 4 + j) * 2));
 #pragma unroll
             for (int p = 0; p < MP; ++p) {
-                f32x4 d = *reinterpret_cast<const f32x4 *>(lds + p * L::PASS + XA_BYTES + (4 * c + j) * 16);
+                f32x4 d = *reinterpret_cast<const f32x4 *>(lds + p * C::PASS + C::XA_BYTES + (4 * c + j) * 16);
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const bf16x8 av = *reinterpret_cast<const bf16x8 *>(lds + a_addr[p] + t * 256);
@@ -174,7 +206,7 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
         }
     }
 
-    // 6. fold the 4 lane groups and the 4 K-slices: RED[wave][lane][pass] = 4 floats
+    // 6. fold lane groups, K-parts and K-slices: RED[wave][lane][pass] = 4 floats
     __syncthreads();  // every wave is done with the operand area, which the partial sums now reuse
     u32x4 *red = reinterpret_cast<u32x4 *>(lds);
 #pragma unroll
@@ -184,58 +216,65 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
         red[(wave * 64 + lane) * MP + p] = v;
     }
     __syncthreads();
-    if (tid < RBW * 16 * 4 * MP) {
-        // tid -> (row block, pass, activation row m, weight row n); n fastest so that stores are contiguous
-        const int n = tid & 15, m = (tid >> 4) & 3, p = (tid >> 6) % MP, rb = tid / (64 * MP);
+    constexpr int UR = C::UR, OUT_PER_UNIT = UR * MPASS * MP;  // weight rows x activation rows (padded to MPASS*MP)
+    if (tid < RBW * OUT_PER_UNIT) {
+        // tid -> (unit, pass, activation row m, weight row n16 of the unit); n16 fastest: contiguous stores
+        const int n16 = tid % UR, m = (tid / UR) % MPASS, p = (tid / (UR * MPASS)) % MP, un = tid / OUT_PER_UNIT;
+        const int rb = n16 / P, rr = n16 % P;
         float t = 0.f;
 #pragma unroll
-        for (int k4 = 0; k4 < 4; ++k4)
+        for (int k4 = 0; k4 < KS; ++k4)
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-                t += reinterpret_cast<const float *>(red)[(((rb * 4 + k4) * 64 + n + 16 * q) * MP + p) * 4 + m];
-        const int nn = (blockIdx.x * RBW + rb) * 16 + n, mm = 4 * p + m;
+            for (int hh = 0; hh < HP; ++hh)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int wsrc = un * 4 + rb * KS + k4, lsrc = 16 * q + hh * P + rr;
+                    t += reinterpret_cast<const float *>(red)[((wsrc * 64 + lsrc) * MP + p) * 4 + hh * MPASS + m];
+                }
+        const int nn = (blockIdx.x * RBW + un) * UR + n16, mm = p * MPASS + m;
         if (nn < N && mm < M) y[(size_t)mm * N + nn] = t;
     }
 }
 
 int gemv_i4g32_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
 
-template <int MT, int RBW>
+template <int MT, int HP, int S, int RBW, int D = 8>
 static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K,
                        hipStream_t st) {
-    typedef GemvLds<(MT + 3) / 4, RBW> L;
+    typedef GemvCfg<MT, HP, S, RBW> C;
     static bool attr_set = false;
     if (!attr_set) {
-        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, RBW>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, L::TOTAL));
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, C::TOTAL));
         attr_set = true;
     }
-    const int rbs = (N + 15) / 16;
-    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, RBW>), dim3((rbs + RBW - 1) / RBW), dim3(256 * RBW), L::TOTAL, st, x,
-                       wp, sc, y, N, K);
+    const int units = (N + C::UR - 1) / C::UR;
+    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D>), dim3((units + RBW - 1) / RBW), dim3(256 * RBW), C::TOTAL,
+                       st, x, wp, sc, y, N, K);
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma launch");
 }
 
 int gemv_i4g32_mfma_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int M, int N, int K,
                              hipStream_t st) {
-    // up to 8 activation rows per launch; more rows reuse the kernel on the next 8
     // the matrix-core kernel wants 16-byte aligned scale rows (K % 256 == 0) and 32-bit byte offsets
     if ((K & 255) != 0 || (int64_t)N * (K / 2) >= ((int64_t)1 << 31) || (reinterpret_cast<uintptr_t>(sc) & 15u) != 0)
         return gemv_i4g32_dispatch(x, wp, sc, y, M, N, K, st);
+    // up to 8 activation rows per launch; more rows reuse the kernel on the next 8
     for (int m0 = 0; m0 < M; m0 += 8) {
         const int mm = (M - m0) < 8 ? (M - m0) : 8;
         const uint16_t *xm = x + (size_t)m0 * K;
         float *ym = y + (size_t)m0 * N;
         int rc = 0;
+        // <rows, K-parts, steps per wave, 4-wave groups per workgroup, prefetch distance>, picked by measurement
         switch (mm) {
-            case 1: rc = launch_mfma<1, 1>(xm, wp, sc, ym, N, K, st); break;
-            case 2: rc = launch_mfma<2, 1>(xm, wp, sc, ym, N, K, st); break;
-            case 3: rc = launch_mfma<3, 1>(xm, wp, sc, ym, N, K, st); break;
-            case 4: rc = launch_mfma<4, 1>(xm, wp, sc, ym, N, K, st); break;
-            case 5: rc = launch_mfma<5, 2>(xm, wp, sc, ym, N, K, st); break;
-            case 6: rc = launch_mfma<6, 2>(xm, wp, sc, ym, N, K, st); break;
-            case 7: rc = launch_mfma<7, 2>(xm, wp, sc, ym, N, K, st); break;
-            default: rc = launch_mfma<8, 2>(xm, wp, sc, ym, N, K, st); break;
+            case 1: rc = launch_mfma<1, 4, 8, 1, 3>(xm, wp, sc, ym, N, K, st); break;
+            case 2: rc = launch_mfma<2, 2, 8, 1, 2>(xm, wp, sc, ym, N, K, st); break;
+            case 3: rc = launch_mfma<3, 1, 8, 1, 8>(xm, wp, sc, ym, N, K, st); break;
+            case 4: rc = launch_mfma<4, 1, 8, 1, 8>(xm, wp, sc, ym, N, K, st); break;
+            case 5: rc = launch_mfma<5, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st); break;
+            case 6: rc = launch_mfma<6, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st); break;
+            case 7: rc = launch_mfma<7, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st); break;
+            default: rc = launch_mfma<8, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st); break;
         }
         if (rc != 0) return rc;
     }
