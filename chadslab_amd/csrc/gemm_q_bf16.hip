@@ -5,15 +5,21 @@
 // Workgroup = 4 waves, output tile 128 x 64, and the four waves split K: wave w owns every fourth slice of
 // K and accumulates a full 128 x 64 partial tile (8 accumulators of v_mfma_f32_32x32x16_bf16).  That choice
 // makes both operands private to a wave:
-//   * B (weights): lane (n = lane%32, kq = lane/32) loads 16 packed bytes of output row n, which is 32 k
-//     (int4, exactly one scale group) or 16 k (int8), dequantises them in registers and feeds them to the
-//     MFMA directly.  Weights never touch LDS.
-//   * A (activations): the wave copies its own 128 x KW slice through a wave-private LDS buffer purely to
-//     transpose from coalesced row-major loads (8 rows x 128 B per instruction) to MFMA fragments.  No other
-//     wave reads it, so the main loop has no barriers.
+//   * B (weights): lane (n = lane%32, kq = lane/32) owns 16 packed bytes of output row n per iteration, which
+//     is 32 k (int4, exactly one scale group) or 16 k (int8).  They arrive by direct global->LDS load in a
+//     wave-private slot, the same lane reads them back, dequantises them in registers (fp16 magic numbers,
+//     one fp32 FMA per element, RNE to bf16) and feeds them to the MFMA.  No other lane ever needs them.
+//   * A (activations): the wave moves its own 128 x KW slice into a wave-private, double-buffered LDS tile with
+//     direct global->LDS loads (global_load_lds_dwordx4: 8 rows x 128 B per instruction, no VGPR round trip),
+//     purely to turn row-major memory into MFMA fragments.  16-byte pieces are XOR-swizzled by row so that
+//     fragment reads are bank-conflict free.  No other wave reads the tile, so the main loop has no barriers.
+//     The tile lives in a ring of eight 32-row slots (two iterations); a slot is refilled for iteration i+2 as
+//     soon as iteration i has consumed it, and the weights of i+1 are dequantised between i's MFMAs.
 // The MFMA k-slot of a lane is free to choose as long as A and B agree: slot group kq covers the kq-th
 // 16-byte weight load, and step t of that load is its t-th 8-k word.
 // The four partial tiles are summed through LDS at the end, rounded to bf16 (RNE) and stored coalesced.
+#include <type_traits>
+
 #include "chadq_common.h"
 
 namespace chadq {
@@ -40,13 +46,15 @@ struct FmtI4G32 {
     typedef uint16_t scale_t;
     // 8 nibbles of word `w` -> 8 bf16 of (u-8)*s, k order.  fp16 magic: 0x6400|u = 1024+u, and a nibble left
     // in bits 7:4 reads as 1024+16u; one fp32 FMA per element removes the offsets and applies the scale.
-    __device__ static __forceinline__ bf16x8 dequant(uint32_t w, float s, float s16, float c0, float c1) {
-        constexpr uint32_t magic = 0x64006400u;
-        const f16x2 h0 = as_f16x2((w & 0x000F000Fu) | magic);  // u0, u4
-        const f16x2 h1 = as_f16x2((w & 0x00F000F0u) | magic);  // 16*u1, 16*u5
+    // mlo = 0x000F000F, mhi = 0x00F000F0 and magic = 0x64006400 are handed over in registers so that each
+    // pair of nibbles costs one v_and_or_b32.
+    __device__ static __forceinline__ bf16x8 dequant(uint32_t w, float s, float s16, float c0, float c1, uint32_t mlo,
+                                                     uint32_t mhi, uint32_t magic) {
+        const f16x2 h0 = as_f16x2(and_or(w, mlo, magic));  // u0, u4
+        const f16x2 h1 = as_f16x2(and_or(w, mhi, magic));  // 16*u1, 16*u5
         const uint32_t w8 = w >> 8;
-        const f16x2 h2 = as_f16x2((w8 & 0x000F000Fu) | magic);  // u2, u6
-        const f16x2 h3 = as_f16x2((w8 & 0x00F000F0u) | magic);  // 16*u3, 16*u7
+        const f16x2 h2 = as_f16x2(and_or(w8, mlo, magic));  // u2, u6
+        const f16x2 h3 = as_f16x2(and_or(w8, mhi, magic));  // 16*u3, 16*u7
         const float f0 = __builtin_fmaf((float)h0.x, s, c0), f4 = __builtin_fmaf((float)h0.y, s, c0);
         const float f1 = __builtin_fmaf((float)h1.x, s16, c1), f5 = __builtin_fmaf((float)h1.y, s16, c1);
         const float f2 = __builtin_fmaf((float)h2.x, s, c0), f6 = __builtin_fmaf((float)h2.y, s, c0);
@@ -77,126 +85,258 @@ struct FmtI8Row {
     }
 };
 
-constexpr int BM = 128, BN = 64, NWAVE = 4;
+constexpr int BM = 128, NWAVE = 4;
 
-template <typename F>
+template <typename F, int NB>
 struct Tile {
+    static constexpr int BN = 32 * NB;              // output columns per workgroup: NB n-blocks of 32
     static constexpr int KL = F::KL;
     static constexpr int KW = 2 * KL;               // k per wave per iteration (two 16-byte loads side by side)
     static constexpr int KIT = NWAVE * KW;          // k per workgroup iteration
     static constexpr int T = KL / 8;                // MFMA steps per 16-byte load
-    static constexpr int ROWB = KW * 2 + 16;        // LDS row pitch in bytes (+16: conflict-free fragment reads)
-    static constexpr int LPR = KW * 2 / 16;         // lanes per activation row in a staging load
-    static constexpr int RPI = 64 / LPR;            // rows per staging instruction
-    static constexpr int NI = BM / RPI;             // staging instructions per iteration
-    static constexpr int STAGE_BYTES = BM * ROWB;   // per wave
+    static constexpr int ROWB = KW * 2;             // LDS row bytes (128 for int4, 64 for int8)
+    static constexpr int PPR = ROWB / 16;           // 16-byte pieces per row (8 or 4)
+    static constexpr int RPL = 8 / PPR;             // rows per 128 bytes of LDS (1 or 2)
+    static constexpr int RPI = 64 / PPR;            // rows per DMA instruction (8 or 16)
+    static constexpr int DPM = 32 / RPI;            // DMA instructions per 32-row m-block (4 or 2)
+    static constexpr int SLOT_BYTES = 32 * ROWB;    // one m-block of one iteration
+    static constexpr int NSLOT = 8;                 // ring: two iterations of four m-blocks
+    static constexpr int A_BYTES = NWAVE * NSLOT * SLOT_BYTES;
+    // weights and scales of one iteration of one wave: NB x 1 KiB (16 B per lane) + NB x 256 B (a dword per lane)
+    static constexpr int BSLOT_BYTES = NB * 1024 + NB * 256;
+    static constexpr int B_OFF = A_BYTES;
+    static constexpr int STAGE_BYTES = A_BYTES + NWAVE * BSLOT_BYTES;
     static constexpr int EPI_BYTES = NWAVE * BM * 32 * 4;
-    static constexpr int LDS_BYTES = (NWAVE * STAGE_BYTES > EPI_BYTES) ? NWAVE * STAGE_BYTES : EPI_BYTES;
+    static constexpr int LDS_BYTES = STAGE_BYTES > EPI_BYTES ? STAGE_BYTES : EPI_BYTES;
 };
 
-template <typename F>
+// 16-byte piece `piece` of row `row` lives in slot piece ^ key(row): fragment reads of 8 consecutive rows
+// then hit 8 different 16-byte bank groups.
+template <typename TL>
+__device__ __forceinline__ int swz(int row, int piece) { return piece ^ ((row / TL::RPL) % TL::PPR); }
+
+// s_waitcnt with only the vector-memory counter set (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);
+}
+
+// GUARD = false assumes K is a multiple of the workgroup's k step (no range checks in the loop).
+template <typename F, int NB, bool GUARD>
 __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__restrict__ x, const void *__restrict__ wq,
                                                           const typename F::scale_t *__restrict__ sc,
                                                           uint16_t *__restrict__ y, int M, int N, int K) {
-    typedef Tile<F> TL;
+    typedef Tile<F, NB> TL;
+    constexpr int BN = TL::BN;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: LDS and global bases stay in SGPRs
     const int nl = lane & 31, kq = lane >> 5;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    uint8_t *stage = lds + wave * TL::STAGE_BYTES;
-    const bool i4 = (TL::KL == 32);
+    // Tile order.  Workgroup i runs on XCD i % 8 (each XCD has its own 4 MiB L2), so tiles are dealt out such
+    // that one XCD walks consecutive n-tiles of the same m-panel: the 128-row activation panel then stays in
+    // that XCD's L2 while the weights stream past, instead of every L2 seeing every panel.
+    const int tiles_n = (N + BN - 1) / BN, tiles = tiles_n * ((M + BM - 1) / BM);
+    const int wg = blockIdx.x, per_xcd = (tiles + 7) / 8;
+    const int tile = (wg % 8) * per_xcd + wg / 8;
+    if (tile >= tiles) return;
+    const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
+    uint8_t *ring = lds + wave * (TL::NSLOT * TL::SLOT_BYTES);
+    constexpr bool i4 = (TL::KL == 32);
     const size_t wrow_bytes = i4 ? (size_t)(K >> 1) : (size_t)K;
     const int G = K >> 5;
 
-    f32x16 acc[4][2];
+    f32x16 acc[4][NB];
 #pragma unroll
     for (int a = 0; a < 4; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < NB; ++b)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
     // weight rows of this lane (clamped so that loads stay in bounds; results for n >= N are never stored)
-    int wr[2];
+    const uint8_t *wbase[NB];
+    const uint16_t *sbase[NB];
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int nb = 0; nb < NB; ++nb) {
         const int n = n0 + nb * 32 + nl;
-        wr[nb] = n < N ? n : N - 1;
+        const int nc = n < N ? n : N - 1;
+        wbase[nb] = (const uint8_t *)wq + (size_t)nc * wrow_bytes;  // row starts; k offsets are added per load
+        sbase[nb] = (const uint16_t *)sc + (size_t)nc * G;
     }
-    // staging coordinates of this lane
-    const int srow = lane / TL::LPR, scol = (lane % TL::LPR) * 8;  // row within an instruction, k offset (elements)
+    // DMA: LDS position lane*16 inside each 1 KiB block is (row dr, slot dslot); the piece that belongs there is
+    // dslot ^ key(row).  Per-lane byte offsets into x are 32-bit (the host checks M*K*2 < 2^32); the k advance
+    // per iteration goes into the scalar base.
+    const int dr = lane / TL::PPR, dslot = lane % TL::PPR;
+    uint32_t doff[4 * TL::DPM], drow[4 * TL::DPM];
+    int dpiece[4 * TL::DPM];
+#pragma unroll
+    for (int i = 0; i < 4 * TL::DPM; ++i) {
+        const int row = i * TL::RPI + dr;
+        const int m = m0 + row < M ? m0 + row : M - 1;
+        dpiece[i] = swz<TL>(row, dslot);
+        drow[i] = (uint32_t)m * (uint32_t)K * 2u;  // byte offset of the row start
+        doff[i] = drow[i] + 16u * dpiece[i];
+    }
+    const uint8_t *xw = reinterpret_cast<const uint8_t *>(x) + (size_t)wave * TL::KW * 2;  // scalar
 
-    u32x4 bq[2];
-    float bs[2];
-    u32x4 ar[TL::NI];
-
-    auto issue_loads = [&](int it) {
+    auto issue_dma = [&](int it, int mb) {
+        const uint8_t *src = xw + (size_t)it * TL::KIT * 2;
+        uint8_t *dst = ring + ((it & 1) * 4 + mb) * TL::SLOT_BYTES;
         const int kb = it * TL::KIT + wave * TL::KW;
-        const int kw = kb + kq * TL::KL;  // first k of this lane's weight load
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-            if (kw < K) {
-                const uint8_t *p = (const uint8_t *)wq + (size_t)wr[nb] * wrow_bytes + (i4 ? (kw >> 1) : kw);
-                bq[nb] = *reinterpret_cast<const u32x4 *>(p);
-                if (i4) bs[nb] = f16_bits_to_f32(((const uint16_t *)sc)[(size_t)wr[nb] * G + (kw >> 5)]);
-            } else {
-                bq[nb] = u32x4{0, 0, 0, 0};
-                bs[nb] = 0.f;
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < TL::NI; ++i) {
-            int m = m0 + i * TL::RPI + srow;
-            m = m < M ? m : M - 1;
-            const int k = kb + scol;
-            ar[i] = (k < K) ? *reinterpret_cast<const u32x4 *>(x + (size_t)m * K + k) : u32x4{0, 0, 0, 0};
+        for (int q = 0; q < TL::DPM; ++q) {
+            const int i = mb * TL::DPM + q;
+            const uint8_t *ptr = src + doff[i];  // = x + (m*K + kb + 8*piece) * 2, inside row m when kb+8*piece < K
+            // columns past K: fetch the start of the row instead (they only ever meet zero weights)
+            if (GUARD && kb + 8 * dpiece[i] >= K) ptr = reinterpret_cast<const uint8_t *>(x) + drow[i];
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)ptr,
+                                             (__attribute__((address_space(3))) void *)(dst + q * 1024), 16, 0, 0);
         }
     };
-    auto store_stage = [&]() {
+    // Weights take the same road: lane (nl, kq) DMAs its 16 packed bytes (and, for int4, its group's scale as
+    // one dword) into a wave-private slot and reads them back itself one iteration later.  With every global
+    // access a DMA, the explicit counts below are the only waits on vector memory in the loop.
+    uint8_t *bslot = lds + TL::B_OFF + wave * TL::BSLOT_BYTES;
+    auto issue_b = [&](int it) {
+        const int kw = it * TL::KIT + wave * TL::KW + kq * TL::KL;  // first k of this lane's 16 bytes
+        const int kc = (!GUARD || kw < K) ? kw : 0;                   // past K: the row start, zeroed on use
 #pragma unroll
-        for (int i = 0; i < TL::NI; ++i)
-            *reinterpret_cast<u32x4 *>(stage + (i * TL::RPI + srow) * TL::ROWB + scol * 2) = ar[i];
+        for (int nb = 0; nb < NB; ++nb) {
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wbase[nb] + (i4 ? kc / 2 : kc)),
+                                             (__attribute__((address_space(3))) void *)(bslot + nb * 1024), 16, 0, 0);
+            if (i4)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(sbase[nb] + (kc >> 5)),
+                                                 (__attribute__((address_space(3))) void *)(bslot + NB * 1024 + nb * 256), 2, 0, 0);
+        }
+    };
+    const uint32_t c_mlo = vgpr_const(0x000F000Fu), c_mhi = vgpr_const(0x00F000F0u), c_magic = vgpr_const(0x64006400u);
+    bf16x8 bf[2][TL::T][NB];  // [set][step][n-block]: dequantised weights of one iteration
+    u32x4 cq[NB];                // the lane's packed weights of the iteration being dequantised
+    float cs[NB][4];             // int4: s, s/16, -1032 s, -72 s
+    auto fetch_b = [&](int it) {  // LDS -> registers, once per iteration; frees the slot for the next request
+        const bool live = !GUARD || ((it * TL::KIT + wave * TL::KW + kq * TL::KL) < K);
+        const uint8_t *src = bslot;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            cq[nb] = *reinterpret_cast<const u32x4 *>(src + nb * 1024 + lane * 16);
+            if constexpr (i4) {
+                const float s = live ? f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(src + NB * 1024 + nb * 256 + lane * 4)) : 0.f;
+                cs[nb][0] = s;
+                cs[nb][1] = s * 0.0625f;
+                cs[nb][2] = -1032.f * s;
+                cs[nb][3] = -72.f * s;
+            } else if (!live) {
+                cq[nb] = u32x4{0, 0, 0, 0};  // int8 zero is the value zero
+            }
+        }
+    };
+    auto dequant_step = [&](int set, int t) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const u32x4 q = cq[nb];
+            if constexpr (i4) {
+                const uint32_t wsel = t == 0 ? q.x : t == 1 ? q.y : t == 2 ? q.z : q.w;
+                bf[set][t][nb] = FmtI4G32::dequant(wsel, cs[nb][0], cs[nb][1], cs[nb][2], cs[nb][3], c_mlo, c_mhi, c_magic);
+            } else {
+                bf[set][t][nb] = t == 0 ? FmtI8Row::dequant(q.x, q.y) : FmtI8Row::dequant(q.z, q.w);
+            }
+        }
     };
 
     const int iters = (K + TL::KIT - 1) / TL::KIT;
-    issue_loads(0);
-    for (int it = 0; it < iters; ++it) {
-        store_stage();
-        const u32x4 cq[2] = {bq[0], bq[1]};
-        const float cs[2] = {bs[0], bs[1]};
-        const bool live = (it * TL::KIT + wave * TL::KW + kq * TL::KL) < K;
-        if (it + 1 < iters) issue_loads(it + 1);
+    constexpr int DPM = TL::DPM, NBL = (i4 ? 2 : 1) * NB, LPI = 4 * DPM + NBL;  // VMEM instructions: m-block, weights, iteration
+    // Request order (memory returns in order, so "X has landed" is "at most so many younger requests are out"):
+    //   prologue   W(0) T(0,0..3) | W(1) T(1,0..3)          W = weights+scales of an iteration, T(i,mb) = m-block
+    //   iteration i issues, after consuming m-block mb, the refill T(i+2,mb); W(i+2) goes out right after the
+    //   first refill, once W(i+1) has been moved from its (single) LDS slot into registers:
+    //              T(i+2,0) W(i+2) T(i+2,1) T(i+2,2) T(i+2,3)
+    // Counts used below are the smallest number of requests that can be younger than the awaited one in any
+    // of these layouts (a smaller count only waits a little longer, never too little).
+    issue_b(0);
 #pragma unroll
-        for (int t = 0; t < TL::T; ++t) {
-            bf16x8 bf[2];
+    for (int mb = 0; mb < 4; ++mb) issue_dma(0, mb);
+    wait_vmcnt<4 * DPM>();  // W(0) is in; T(0,*) may still be out
+    fetch_b(0);
+    if (iters > 1) {
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the slot has been read before it is requested again
+        issue_b(1);
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
-                if constexpr (TL::KL == 32) {
-                    const float s = cs[nb];
-                    const uint32_t wsel = t == 0 ? cq[nb].x : t == 1 ? cq[nb].y : t == 2 ? cq[nb].z : cq[nb].w;
-                    bf[nb] = FmtI4G32::dequant(wsel, s, s * 0.0625f, -1032.f * s, -72.f * s);
-                } else {
-                    bf[nb] = t == 0 ? FmtI8Row::dequant(cq[nb].x, cq[nb].y) : FmtI8Row::dequant(cq[nb].z, cq[nb].w);
-                    if (!live) {
-                        const u32x4 z = {0, 0, 0, 0};
-                        __builtin_memcpy(&bf[nb], &z, 16);
+        for (int mb = 0; mb < 4; ++mb) issue_dma(1, mb);
+    }
+#pragma unroll
+    for (int t = 0; t < TL::T; ++t) dequant_step(0, t);
+
+    auto iteration = [&](int it, auto set_c, auto more1_c, auto more2_c) {
+        constexpr int set = decltype(set_c)::value;
+        constexpr bool more1 = decltype(more1_c)::value, more2 = decltype(more2_c)::value;  // it+1 / it+2 exist
+        const uint8_t *abase = ring + set * 4 * TL::SLOT_BYTES;
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) {
+            // T(it, mb) has landed
+            if (more2) {
+                if (mb == 0) wait_vmcnt<3 * DPM + LPI>();
+                else wait_vmcnt<3 * DPM + LPI + NBL>();
+            } else if (more1) {
+                if (mb == 0) wait_vmcnt<3 * DPM + LPI>();
+                if (mb == 1) wait_vmcnt<2 * DPM + LPI>();
+                if (mb == 2) wait_vmcnt<1 * DPM + LPI>();
+                if (mb == 3) wait_vmcnt<LPI>();
+            } else {
+                if (mb == 0) wait_vmcnt<3 * DPM>();
+                if (mb == 1) wait_vmcnt<2 * DPM>();
+                if (mb == 2) wait_vmcnt<1 * DPM>();
+                if (mb == 3) wait_vmcnt<0>();
+            }
+            const uint8_t *ab = abase + mb * TL::SLOT_BYTES;
+#pragma unroll
+            for (int t = 0; t < TL::T; ++t) {
+                const bf16x8 af = *reinterpret_cast<const bf16x8 *>(ab + nl * TL::ROWB + swz<TL>(nl, kq * TL::T + t) * 16);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                    acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bf[set][t][nb], acc[mb][nb], 0, 0, 0);
+            }
+            if (more2) issue_dma(it + 2, mb);  // the slot just consumed
+            // next iteration's weights become MFMA operands while this iteration's MFMAs run
+            if (more1) {
+                if (mb == 0) {
+                    // W(it+1) has landed: younger are T(it+1,1..3) and, if issued, the refill above
+                    if (more2) wait_vmcnt<4 * DPM>();
+                    else wait_vmcnt<3 * DPM>();
+                    fetch_b(it + 1);
+                    if (more2) {
+                        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): read out before it is requested again
+                        issue_b(it + 2);
                     }
                 }
-            }
-#pragma unroll
-            for (int mb = 0; mb < 4; ++mb) {
-                const bf16x8 af = *reinterpret_cast<const bf16x8 *>(stage + (mb * 32 + nl) * TL::ROWB + (kq * TL::KL + 8 * t) * 2);
-#pragma unroll
-                for (int nb = 0; nb < 2; ++nb)
-                    acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bf[nb], acc[mb][nb], 0, 0, 0);
+                if (mb < TL::T) dequant_step(set ^ 1, mb);
             }
         }
+    };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    int it = 0;
+    for (; it + 3 < iters; it += 2) {  // steady state: no conditions inside, so the scheduler sees one block
+        iteration(it, S0{}, std::true_type{}, std::true_type{});
+        iteration(it + 1, S1{}, std::true_type{}, std::true_type{});
+    }
+    // the last one to three iterations (it is even here)
+    const int left = iters - it;
+    if (left == 3) {
+        iteration(it, S0{}, std::true_type{}, std::true_type{});
+        iteration(it + 1, S1{}, std::true_type{}, std::false_type{});
+        iteration(it + 2, S0{}, std::false_type{}, std::false_type{});
+    } else if (left == 2) {
+        iteration(it, S0{}, std::true_type{}, std::false_type{});
+        iteration(it + 1, S1{}, std::false_type{}, std::false_type{});
+    } else if (left == 1) {
+        iteration(it, S0{}, std::false_type{}, std::false_type{});
     }
 
     // cross-wave sum, one 128 x 32 half tile at a time: [wave][row][32] fp32 in LDS
-    float rs[2] = {1.f, 1.f};
+    const bool y_vec = ((N & 3) == 0) && ((reinterpret_cast<uintptr_t>(y) & 7u) == 0);
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int nb = 0; nb < NB; ++nb) {
         __syncthreads();
         float *red = reinterpret_cast<float *>(lds) + wave * (BM * 32);
 #pragma unroll
@@ -218,7 +358,7 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
                 s += *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(lds) + w2 * (BM * 32) + row * 32 + c4);
             const int m = m0 + row, n = n0 + nb * 32 + c4;
             if (m < M) {
-                if constexpr (TL::KL == 16) {
+                if constexpr (!i4) {
                     const float *scf = (const float *)sc;
                     s.x *= (n + 0 < N) ? scf[n + 0] : 0.f;
                     s.y *= (n + 1 < N) ? scf[n + 1] : 0.f;
@@ -226,7 +366,7 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
                     s.w *= (n + 3 < N) ? scf[n + 3] : 0.f;
                 }
                 uint16_t *yp = y + (size_t)m * N + n;
-                if (n + 3 < N && ((N & 3) == 0)) {
+                if (n + 3 < N && y_vec) {
                     u32x2 o = {pack_bf16_rne(s.x, s.y), pack_bf16_rne(s.z, s.w)};
                     *reinterpret_cast<u32x2 *>(yp) = o;
                 } else {
@@ -237,22 +377,34 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
             }
         }
     }
-    (void)rs;
+}
+
+template <typename F, int NB, bool GUARD>
+static int launch_gemm_g(const uint16_t *x, const void *wq, const typename F::scale_t *sc, uint16_t *y, int M, int N,
+                         int K, hipStream_t st) {
+    typedef Tile<F, NB> TL;
+    static bool attr_set = false;
+    if (!attr_set) {
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q_bf16_kernel<F, NB, GUARD>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, TL::LDS_BYTES));
+        attr_set = true;
+    }
+    const int tiles = ((N + TL::BN - 1) / TL::BN) * ((M + BM - 1) / BM);
+    const int grid = ((tiles + 7) / 8) * 8;  // a multiple of the 8 XCDs; surplus workgroups exit at once
+    hipLaunchKernelGGL((gemm_q_bf16_kernel<F, NB, GUARD>), dim3(grid), dim3(256), TL::LDS_BYTES, st, x, wq, sc, y, M, N, K);
+    return hip_check(hipGetLastError(), "gemm_q_bf16 launch");
 }
 
 template <typename F>
 static int launch_gemm(const uint16_t *x, const void *wq, const typename F::scale_t *sc, uint16_t *y, int M, int N,
                        int K, hipStream_t st) {
-    typedef Tile<F> TL;
-    static bool attr_set = false;
-    if (!attr_set) {
-        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q_bf16_kernel<F>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, TL::LDS_BYTES));
-        attr_set = true;
-    }
-    dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
-    hipLaunchKernelGGL((gemm_q_bf16_kernel<F>), grid, dim3(256), TL::LDS_BYTES, st, x, wq, sc, y, M, N, K);
-    return hip_check(hipGetLastError(), "gemm_q_bf16 launch");
+    CHADQ_REQUIRE((int64_t)M * K * 2 < ((int64_t)1 << 32), CHADQ_ERR_SHAPE,
+                  "gemm: activations of %d x %d exceed the 4 GiB the kernel's 32-bit offsets cover", M, K);
+    // NB = 2 (128 x 64 tiles).  The kernel is written for any NB; NB = 4 halves the traffic on the activation
+    // panel but needs 256 accumulator registers plus two sets of dequantised operands and spills, so it is
+    // not instantiated.
+    if (K % Tile<F, 2>::KIT != 0) return launch_gemm_g<F, 2, true>(x, wq, sc, y, M, N, K, st);
+    return launch_gemm_g<F, 2, false>(x, wq, sc, y, M, N, K, st);
 }
 
 int gemm_i4g32_bf16_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, uint16_t *y, int M, int N,
