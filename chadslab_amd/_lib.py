@@ -6,7 +6,7 @@ There is no CPU or PyTorch fallback.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_int, c_int64, c_void_p
+from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libchadq.so"
@@ -24,7 +24,16 @@ SIGNATURES = {
     "chadq_gemv_i8row": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "chadq_gemm_i4g32_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "chadq_gemm_i8row_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "chadq_moe_route": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "chadq_moe_ffn_i4g32_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "chadq_moe_ffn_i4g32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_void_p, c_size_t, c_void_p]),
 }
+
+
+class MoeExpertI4G32(ctypes.Structure):
+    """Mirror of chadq_moe_expert_i4g32: six device pointers."""
+    _fields_ = [(n, c_void_p) for n in ("wg", "sg", "wu", "su", "wd", "sd")]
 
 _STATUS_EXC = {-1: ValueError, -2: ValueError, -3: ValueError, -4: ValueError, -5: RuntimeError, -6: RuntimeError}
 

@@ -51,6 +51,11 @@ int gemm_i4g32_bf16_dispatch(const uint16_t *, const uint8_t *, const uint16_t *
 int gemm_i8row_bf16_dispatch(const uint16_t *, const int8_t *, const float *, uint16_t *, int, int, int,
                              hipStream_t);
 
+size_t moe_workspace_bytes(int, int, int, int, int);
+int moe_route_launch(const float *, int32_t *, float *, int, int, int, int, hipStream_t);
+int moe_ffn_i4g32_launch(const uint16_t *, const float *, const chadq_moe_expert_i4g32 *, uint16_t *, int, int, int, int, int,
+                         int, void *, hipStream_t);
+
 }  // namespace chadq
 
 using namespace chadq;
@@ -146,6 +151,44 @@ int chadq_gemm_i8row_bf16(const uint16_t *x_bf16, const int8_t *w8, const float 
     CHADQ_REQUIRE(x_bf16 && w8 && scale && y_bf16, CHADQ_ERR_NULL, "chadq_gemm_i8row_bf16: null pointer");
     CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(w8), CHADQ_ERR_ALIGN, "chadq_gemm_i8row_bf16: x and w8 must be 16-byte aligned");
     return gemm_i8row_bf16_dispatch(x_bf16, w8, scale, y_bf16, M, N, K, st);
+}
+
+static bool moe_sizes_ok(int T, int H, int F, int E, int top_k) {
+    return T >= 1 && H >= 32 && F >= 32 && H % 32 == 0 && F % 32 == 0 && E >= 1 && E <= 16 && top_k >= 1 && top_k <= 8 &&
+           top_k <= E;
+}
+
+int chadq_moe_route(const float *logits, int32_t *idx, float *w, int T, int E, int top_k, int renorm, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(T >= 0 && E >= 1 && E <= 16 && top_k >= 1 && top_k <= 8 && top_k <= E, CHADQ_ERR_SHAPE,
+                  "chadq_moe_route: T=%d E=%d top_k=%d (E <= 16, top_k <= min(E, 8))", T, E, top_k);
+    if (T == 0) return 0;
+    CHADQ_REQUIRE(logits && idx && w, CHADQ_ERR_NULL, "chadq_moe_route: null pointer");
+    return moe_route_launch(logits, idx, w, T, E, top_k, renorm, st);
+}
+
+size_t chadq_moe_ffn_i4g32_workspace_bytes(int T, int H, int F, int E, int top_k) {
+    if (!moe_sizes_ok(T, H, F, E, top_k)) return 0;
+    return moe_workspace_bytes(T, H, F, E, top_k);
+}
+
+int chadq_moe_ffn_i4g32(const uint16_t *x_bf16, const float *logits, const chadq_moe_expert_i4g32 *experts,
+                        uint16_t *y_bf16, int T, int H, int F, int E, int top_k, int renorm, void *workspace,
+                        size_t workspace_bytes, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(moe_sizes_ok(T, H, F, E, top_k), CHADQ_ERR_SHAPE,
+                  "chadq_moe_ffn_i4g32: T=%d H=%d F=%d E=%d top_k=%d (H, F multiples of 32; E <= 16; top_k <= min(E, 8))", T,
+                  H, F, E, top_k);
+    CHADQ_REQUIRE(x_bf16 && logits && experts && y_bf16, CHADQ_ERR_NULL, "chadq_moe_ffn_i4g32: null pointer");
+    for (int e = 0; e < E; ++e)
+        CHADQ_REQUIRE(experts[e].wg && experts[e].sg && experts[e].wu && experts[e].su && experts[e].wd && experts[e].sd,
+                      CHADQ_ERR_NULL, "chadq_moe_ffn_i4g32: expert %d has a null weight pointer", e);
+    const size_t need = moe_workspace_bytes(T, H, F, E, top_k);
+    CHADQ_REQUIRE(workspace && workspace_bytes >= need, CHADQ_ERR_WORKSPACE,
+                  "chadq_moe_ffn_i4g32: workspace of %zu bytes needed, %zu given", need, workspace ? workspace_bytes : (size_t)0);
+    CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(workspace) && aligned16(y_bf16), CHADQ_ERR_ALIGN,
+                  "chadq_moe_ffn_i4g32: x, y and workspace must be 16-byte aligned");
+    return moe_ffn_i4g32_launch(x_bf16, logits, experts, y_bf16, T, H, F, E, top_k, renorm, workspace, st);
 }
 
 }  // extern "C"

@@ -38,6 +38,16 @@ int check_device();
         if (!(cond)) return ::chadq::fail((code), __VA_ARGS__); \
     } while (0)
 
+// One member of a grouped GEMM launch (device memory): y[M,N] = x[M,K] * w[N,K]^T with int4 group-32 weights.
+struct GemmGroup {
+    const uint16_t *x;  // bf16 [M,K]
+    const void *w;      // packed weights [N,K/2]
+    const void *sc;     // fp16 scales [N,K/32]
+    void *y;            // bf16 or fp32 [M,N]
+    int M;
+    int pad;
+};
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ---- device side ------------------------------------------------------------------------------

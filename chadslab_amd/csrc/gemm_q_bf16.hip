@@ -123,11 +123,23 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 // GUARD = false assumes K is a multiple of the workgroup's k step (no range checks in the loop).
-template <typename F, int NB, bool GUARD>
+// OUTF32: y is fp32 [M,N] instead of bf16.  groups != nullptr: grouped launch, blockIdx.y selects a descriptor
+// (activations, weights, output and row count of one group; N and K are common) - this is how the MoE expert
+// GEMMs run as one launch over experts whose row counts only the GPU knows.
+template <typename F, int NB, bool GUARD, bool OUTF32>
 __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__restrict__ x, const void *__restrict__ wq,
                                                           const typename F::scale_t *__restrict__ sc,
-                                                          uint16_t *__restrict__ y, int M, int N, int K) {
+                                                          uint16_t *__restrict__ y, int M, int N, int K,
+                                                          const GemmGroup *__restrict__ groups) {
     typedef Tile<F, NB> TL;
+    if (groups) {
+        const GemmGroup g = groups[blockIdx.y];
+        x = g.x;
+        wq = g.w;
+        sc = reinterpret_cast<const typename F::scale_t *>(g.sc);
+        y = reinterpret_cast<uint16_t *>(g.y);
+        M = g.M;
+    }
     constexpr int BN = TL::BN;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -334,7 +346,7 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
     }
 
     // cross-wave sum, one 128 x 32 half tile at a time: [wave][row][32] fp32 in LDS
-    const bool y_vec = ((N & 3) == 0) && ((reinterpret_cast<uintptr_t>(y) & 7u) == 0);
+    const bool y_vec = ((N & 3) == 0) && ((reinterpret_cast<uintptr_t>(y) & 15u) == 0);
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         __syncthreads();
@@ -365,56 +377,73 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
                     s.z *= (n + 2 < N) ? scf[n + 2] : 0.f;
                     s.w *= (n + 3 < N) ? scf[n + 3] : 0.f;
                 }
-                uint16_t *yp = y + (size_t)m * N + n;
-                if (n + 3 < N && y_vec) {
-                    u32x2 o = {pack_bf16_rne(s.x, s.y), pack_bf16_rne(s.z, s.w)};
-                    *reinterpret_cast<u32x2 *>(yp) = o;
+                if constexpr (OUTF32) {
+                    float *yp = reinterpret_cast<float *>(y) + (size_t)m * N + n;
+                    if (n + 3 < N && y_vec) {
+                        *reinterpret_cast<f32x4 *>(yp) = s;
+                    } else {
+                        const float sv[4] = {s.x, s.y, s.z, s.w};
+                        for (int j = 0; j < 4; ++j)
+                            if (n + j < N) yp[j] = sv[j];
+                    }
                 } else {
-                    const float sv[4] = {s.x, s.y, s.z, s.w};
-                    for (int j = 0; j < 4; ++j)
-                        if (n + j < N) yp[j] = (uint16_t)f32_to_bf16_bits(sv[j]);
+                    uint16_t *yp = y + (size_t)m * N + n;
+                    if (n + 3 < N && y_vec) {
+                        u32x2 o = {pack_bf16_rne(s.x, s.y), pack_bf16_rne(s.z, s.w)};
+                        *reinterpret_cast<u32x2 *>(yp) = o;
+                    } else {
+                        const float sv[4] = {s.x, s.y, s.z, s.w};
+                        for (int j = 0; j < 4; ++j)
+                            if (n + j < N) yp[j] = (uint16_t)f32_to_bf16_bits(sv[j]);
+                    }
                 }
             }
         }
     }
 }
 
-template <typename F, int NB, bool GUARD>
-static int launch_gemm_g(const uint16_t *x, const void *wq, const typename F::scale_t *sc, uint16_t *y, int M, int N,
-                         int K, hipStream_t st) {
+template <typename F, int NB, bool GUARD, bool OUTF32>
+static int launch_gemm_g(const uint16_t *x, const void *wq, const typename F::scale_t *sc, void *y, int M, int N,
+                         int K, const GemmGroup *groups, int ngroups, hipStream_t st) {
     typedef Tile<F, NB> TL;
     static bool attr_set = false;
     if (!attr_set) {
-        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q_bf16_kernel<F, NB, GUARD>),
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q_bf16_kernel<F, NB, GUARD, OUTF32>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, TL::LDS_BYTES));
         attr_set = true;
     }
-    const int tiles = ((N + TL::BN - 1) / TL::BN) * ((M + BM - 1) / BM);
+    const int tiles = ((N + TL::BN - 1) / TL::BN) * ((M + BM - 1) / BM);  // M = the largest group in a grouped launch
     const int grid = ((tiles + 7) / 8) * 8;  // a multiple of the 8 XCDs; surplus workgroups exit at once
-    hipLaunchKernelGGL((gemm_q_bf16_kernel<F, NB, GUARD>), dim3(grid), dim3(256), TL::LDS_BYTES, st, x, wq, sc, y, M, N, K);
+    hipLaunchKernelGGL((gemm_q_bf16_kernel<F, NB, GUARD, OUTF32>), dim3(grid, groups ? ngroups : 1), dim3(256),
+                       TL::LDS_BYTES, st, x, wq, sc, reinterpret_cast<uint16_t *>(y), M, N, K, groups);
     return hip_check(hipGetLastError(), "gemm_q_bf16 launch");
 }
 
-template <typename F>
-static int launch_gemm(const uint16_t *x, const void *wq, const typename F::scale_t *sc, uint16_t *y, int M, int N,
-                       int K, hipStream_t st) {
+// NB = 2 (128 x 64 tiles).  The kernel is written for any NB; NB = 4 halves the traffic on the activation panel
+// but needs 256 accumulator registers plus two sets of dequantised operands and spills, so it is not instantiated.
+template <typename F, bool OUTF32>
+static int launch_gemm(const uint16_t *x, const void *wq, const typename F::scale_t *sc, void *y, int M, int N, int K,
+                       const GemmGroup *groups, int ngroups, hipStream_t st) {
     CHADQ_REQUIRE((int64_t)M * K * 2 < ((int64_t)1 << 32), CHADQ_ERR_SHAPE,
                   "gemm: activations of %d x %d exceed the 4 GiB the kernel's 32-bit offsets cover", M, K);
-    // NB = 2 (128 x 64 tiles).  The kernel is written for any NB; NB = 4 halves the traffic on the activation
-    // panel but needs 256 accumulator registers plus two sets of dequantised operands and spills, so it is
-    // not instantiated.
-    if (K % Tile<F, 2>::KIT != 0) return launch_gemm_g<F, 2, true>(x, wq, sc, y, M, N, K, st);
-    return launch_gemm_g<F, 2, false>(x, wq, sc, y, M, N, K, st);
+    if (K % Tile<F, 2>::KIT != 0) return launch_gemm_g<F, 2, true, OUTF32>(x, wq, sc, y, M, N, K, groups, ngroups, st);
+    return launch_gemm_g<F, 2, false, OUTF32>(x, wq, sc, y, M, N, K, groups, ngroups, st);
 }
 
 int gemm_i4g32_bf16_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, uint16_t *y, int M, int N,
                              int K, hipStream_t st) {
-    return launch_gemm<FmtI4G32>(x, wp, sc, y, M, N, K, st);
+    return launch_gemm<FmtI4G32, false>(x, wp, sc, y, M, N, K, nullptr, 0, st);
 }
 
 int gemm_i8row_bf16_dispatch(const uint16_t *x, const int8_t *w8, const float *sc, uint16_t *y, int M, int N, int K,
                              hipStream_t st) {
-    return launch_gemm<FmtI8Row>(x, w8, sc, y, M, N, K, st);
+    return launch_gemm<FmtI8Row, false>(x, w8, sc, y, M, N, K, nullptr, 0, st);
+}
+
+// One launch over `ngroups` int4 group-32 products that share N and K; m_max bounds every group's row count.
+int gemm_i4g32_grouped(const GemmGroup *groups, int ngroups, int m_max, int N, int K, bool out_f32, hipStream_t st) {
+    if (out_f32) return launch_gemm<FmtI4G32, true>(nullptr, nullptr, nullptr, nullptr, m_max, N, K, groups, ngroups, st);
+    return launch_gemm<FmtI4G32, false>(nullptr, nullptr, nullptr, nullptr, m_max, N, K, groups, ngroups, st);
 }
 
 }  // namespace chadq

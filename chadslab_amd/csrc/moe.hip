@@ -1,0 +1,230 @@
+// Mixture-of-experts FFN on int4 group-32 expert weights (benchmark config 3):
+//   p = softmax(logits[t,:]);  the top_k experts of token t by logit (lowest index wins ties), weights p
+//   renormalised to sum 1 if asked;  y[t] = bf16( sum_j w[t,j] * down_e( bf16( silu(gate_e x_t) * (up_e x_t) ) ) ).
+//
+// Everything runs on the caller's stream without a host round trip: the router kernel also sorts the
+// (token, slot) pairs by expert (stable: by pair index inside an expert) and writes the per-expert descriptors
+// of three grouped GEMM launches (gate, up: fp32 out; down: fp32 out), whose row counts therefore never
+// leave the GPU.  Gate/up/down are the dequant-GEMM kernel in grouped mode; the small kernels here are the
+// gather, the SiLU gate and the weighted combine.
+#include "chadq_common.h"
+
+namespace chadq {
+
+constexpr int MOE_MAX_E = 16;
+constexpr int MOE_MAX_K = 8;
+
+struct MoeExperts {  // by value in the kernel arguments
+    const void *wg[MOE_MAX_E], *sg[MOE_MAX_E], *wu[MOE_MAX_E], *su[MOE_MAX_E], *wd[MOE_MAX_E], *sd[MOE_MAX_E];
+};
+
+struct MoeWs {  // workspace carved up on the host
+    int32_t *idx;        // [T,top_k] expert of each pair
+    float *w;            // [T,top_k] routing weight of each pair
+    int32_t *pos;        // [P] row of the pair in expert-sorted order
+    int32_t *tok;        // [P] token of the sorted row
+    int32_t *cnt;        // [E] rows per expert, then [E] offsets
+    GemmGroup *groups;   // [3*E] gate, up, down
+    uint16_t *xs;        // [P,H] gathered activations (bf16)
+    float *g, *u;        // [P,F]
+    uint16_t *h;         // [P,F] bf16
+    float *yp;           // [P,H]
+};
+
+int gemm_i4g32_grouped(const GemmGroup *groups, int ngroups, int m_max, int N, int K, bool out_f32, hipStream_t st);
+
+// One workgroup.  Phase 1: softmax + top-k per token.  Phase 2: stable counting sort of the pairs by expert.
+// Phase 3: descriptors.  idx/w may be the caller's arrays (chadq_moe_route) with everything else null.
+__global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict__ logits, int32_t *__restrict__ idx,
+                                                         float *__restrict__ w, int T, int E, int top_k, int renorm,
+                                                         MoeWs ws, MoeExperts ex, int H, int F) {
+    __shared__ int s_base[MOE_MAX_E];   // rows of expert e seen so far
+    __shared__ int s_wave[16];          // per-wave counts of the current expert in the current chunk
+    __shared__ int s_off[MOE_MAX_E + 1];
+    const int tid = threadIdx.x, B = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = B >> 6;
+    if (tid < MOE_MAX_E) s_base[tid] = 0;
+
+    for (int t = tid; t < T; t += B) {
+        const float *z = logits + (size_t)t * E;
+        float mx = z[0];
+        for (int e = 1; e < E; ++e) mx = fmaxf(mx, z[e]);
+        float sum = 0.f;
+        for (int e = 0; e < E; ++e) sum += __expf(z[e] - mx);
+        int chosen[MOE_MAX_K];
+        float pw[MOE_MAX_K], wsum = 0.f;
+        for (int j = 0; j < top_k; ++j) {
+            int best = -1;
+            for (int e = 0; e < E; ++e) {
+                bool taken = false;
+                for (int i = 0; i < j; ++i) taken |= (chosen[i] == e);
+                if (!taken && (best < 0 || z[e] > z[best])) best = e;  // strict >: the lowest index wins ties
+            }
+            chosen[j] = best;
+            pw[j] = __expf(z[best] - mx) / sum;
+            wsum += pw[j];
+        }
+        for (int j = 0; j < top_k; ++j) {
+            idx[(size_t)t * top_k + j] = chosen[j];
+            w[(size_t)t * top_k + j] = renorm ? pw[j] / wsum : pw[j];
+        }
+    }
+    if (!ws.pos) return;  // routing only
+    __syncthreads();      // idx (global) written by this workgroup is visible to it after the barrier
+
+    const int P = T * top_k;
+    for (int c0 = 0; c0 < P; c0 += B) {
+        const int p = c0 + tid;
+        const int e_mine = p < P ? idx[p] : -1;
+        int rank = 0;
+        for (int e = 0; e < E; ++e) {
+            const bool flag = (e_mine == e);
+            const unsigned long long m = __ballot(flag);
+            const int below = __popcll(m & ((1ull << lane) - 1ull));
+            if (lane == 0) s_wave[wave] = __popcll(m);
+            __syncthreads();
+            int woff = 0, total = 0;
+            for (int i = 0; i < nw; ++i) {
+                const int c = s_wave[i];
+                woff += (i < wave) ? c : 0;
+                total += c;
+            }
+            if (flag) rank = s_base[e] + woff + below;
+            __syncthreads();
+            if (tid == 0) s_base[e] += total;
+            __syncthreads();
+        }
+        if (p < P) ws.pos[p] = rank;  // rank inside its expert for now
+    }
+    if (tid == 0) {
+        int o = 0;
+        for (int e = 0; e < E; ++e) {
+            s_off[e] = o;
+            ws.cnt[e] = s_base[e];
+            ws.cnt[E + e] = o;
+            o += s_base[e];
+        }
+        s_off[E] = o;
+    }
+    __syncthreads();
+    for (int p = tid; p < P; p += B) {
+        const int row = s_off[idx[p]] + ws.pos[p];
+        ws.pos[p] = row;
+        ws.tok[row] = p / top_k;
+    }
+    if (tid < E) {
+        const int e = tid, o = s_off[e], m = s_base[e];
+        ws.groups[e] = GemmGroup{ws.xs + (size_t)o * H, ex.wg[e], ex.sg[e], ws.g + (size_t)o * F, m, 0};
+        ws.groups[E + e] = GemmGroup{ws.xs + (size_t)o * H, ex.wu[e], ex.su[e], ws.u + (size_t)o * F, m, 0};
+        ws.groups[2 * E + e] = GemmGroup{ws.h + (size_t)o * F, ex.wd[e], ex.sd[e], ws.yp + (size_t)o * H, m, 0};
+    }
+}
+
+// xs[row] = x[tok[row]]; one 16-byte piece per thread
+__global__ __launch_bounds__(256) void moe_gather_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ tok,
+                                                         uint16_t *__restrict__ xs, int P, int H) {
+    const int pieces = H / 8;
+    const int64_t total = (int64_t)P * pieces, stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int row = (int)(i / pieces), c = (int)(i % pieces);
+        reinterpret_cast<u32x4 *>(xs)[i] = reinterpret_cast<const u32x4 *>(x + (size_t)tok[row] * H)[c];
+    }
+}
+
+// h = bf16( silu(g) * u ), 4 elements per thread
+__global__ __launch_bounds__(256) void moe_act_kernel(const float *__restrict__ g, const float *__restrict__ u,
+                                                      uint16_t *__restrict__ h, int64_t n4) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+        const f32x4 a = reinterpret_cast<const f32x4 *>(g)[i], b = reinterpret_cast<const f32x4 *>(u)[i];
+        float r[4];
+        const float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r[j] = av[j] / (1.f + __expf(-av[j])) * bv[j];
+        u32x2 o = {f32_to_bf16_bits(r[0]) | (f32_to_bf16_bits(r[1]) << 16), f32_to_bf16_bits(r[2]) | (f32_to_bf16_bits(r[3]) << 16)};
+        reinterpret_cast<u32x2 *>(h)[i] = o;
+    }
+}
+
+// y[t] = bf16( sum_j w[t,j] * yp[pos[t*top_k+j]] ), slots in order; 4 columns per thread
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restrict__ yp, const int32_t *__restrict__ pos,
+                                                          const float *__restrict__ w, uint16_t *__restrict__ y, int T,
+                                                          int H, int top_k) {
+    const int q = H / 4;
+    const int64_t total = (int64_t)T * q, stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int t = (int)(i / q), c = (int)(i % q);
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < top_k; ++j) {
+            const f32x4 v = reinterpret_cast<const f32x4 *>(yp + (size_t)pos[t * top_k + j] * H)[c];
+            acc += v * w[t * top_k + j];
+        }
+        u32x2 o = {f32_to_bf16_bits(acc.x) | (f32_to_bf16_bits(acc.y) << 16), f32_to_bf16_bits(acc.z) | (f32_to_bf16_bits(acc.w) << 16)};
+        reinterpret_cast<u32x2 *>(y)[i] = o;
+    }
+}
+
+static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// carve-up of the workspace; base == nullptr just measures
+static size_t moe_layout(uint8_t *base, int T, int H, int F, int E, int top_k, MoeWs *ws) {
+    const size_t P = (size_t)T * top_k;
+    size_t o = 0;
+    auto take = [&](size_t bytes) {
+        uint8_t *p = base ? base + o : nullptr;
+        o += align_up(bytes);
+        return p;
+    };
+    MoeWs w;
+    w.idx = (int32_t *)take(P * 4);
+    w.w = (float *)take(P * 4);
+    w.pos = (int32_t *)take(P * 4);
+    w.tok = (int32_t *)take(P * 4);
+    w.cnt = (int32_t *)take((size_t)2 * E * 4);
+    w.groups = (GemmGroup *)take((size_t)3 * E * sizeof(GemmGroup));
+    w.xs = (uint16_t *)take(P * H * 2);
+    w.g = (float *)take(P * F * 4);
+    w.u = (float *)take(P * F * 4);
+    w.h = (uint16_t *)take(P * F * 2);
+    w.yp = (float *)take(P * H * 4);
+    if (ws) *ws = w;
+    return o;
+}
+
+size_t moe_workspace_bytes(int T, int H, int F, int E, int top_k) { return moe_layout(nullptr, T, H, F, E, top_k, nullptr); }
+
+int moe_route_launch(const float *logits, int32_t *idx, float *w, int T, int E, int top_k, int renorm, hipStream_t st) {
+    MoeWs ws = {};
+    MoeExperts ex = {};
+    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 0, st, logits, idx, w, T, E, top_k, renorm, ws, ex, 0, 0);
+    return hip_check(hipGetLastError(), "moe_route launch");
+}
+
+int moe_ffn_i4g32_launch(const uint16_t *x, const float *logits, const chadq_moe_expert_i4g32 *experts, uint16_t *y,
+                         int T, int H, int F, int E, int top_k, int renorm, void *workspace, hipStream_t st) {
+    MoeWs ws;
+    moe_layout(reinterpret_cast<uint8_t *>(workspace), T, H, F, E, top_k, &ws);
+    MoeExperts ex = {};
+    for (int e = 0; e < E; ++e) {
+        ex.wg[e] = experts[e].wg;
+        ex.sg[e] = experts[e].sg;
+        ex.wu[e] = experts[e].wu;
+        ex.su[e] = experts[e].su;
+        ex.wd[e] = experts[e].wd;
+        ex.sd[e] = experts[e].sd;
+    }
+    const int P = T * top_k;
+    const int m_max = P < T ? P : T;  // an expert gets a token at most once
+    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 0, st, logits, ws.idx, ws.w, T, E, top_k, renorm, ws, ex, H, F);
+    hipLaunchKernelGGL(moe_gather_kernel, dim3(512), dim3(256), 0, st, x, ws.tok, ws.xs, P, H);
+    int rc = hip_check(hipGetLastError(), "moe route/gather launch");
+    if (rc) return rc;
+    rc = gemm_i4g32_grouped(ws.groups, 2 * E, m_max, F, H, true, st);  // gate and up: fp32 [P,F] each
+    if (rc) return rc;
+    hipLaunchKernelGGL(moe_act_kernel, dim3(2048), dim3(256), 0, st, ws.g, ws.u, ws.h, (int64_t)P * F / 4);
+    rc = gemm_i4g32_grouped(ws.groups + 2 * E, E, m_max, H, F, true, st);  // down: fp32 [P,H]
+    if (rc) return rc;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(1024), dim3(256), 0, st, ws.yp, ws.pos, ws.w, y, T, H, top_k);
+    return hip_check(hipGetLastError(), "moe act/combine launch");
+}
+
+}  // namespace chadq

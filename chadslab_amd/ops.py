@@ -125,3 +125,51 @@ def qlinear(x: torch.Tensor, qw: QWeight, *, out_dtype: Optional[torch.dtype] = 
     if out_dtype is not None and y.dtype != out_dtype:
         y = y.to(out_dtype)
     return y.reshape(*lead, qw.N)
+
+
+def moe_route(logits: torch.Tensor, top_k: int = 2, renorm: bool = True):
+    """softmax over experts, top_k by logit (lowest index wins ties) -> (idx int32 [T,top_k], w fp32 [T,top_k])."""
+    z = _dev(logits, "logits", torch.float32)
+    t, e = z.shape
+    idx = torch.empty(t, top_k, dtype=torch.int32, device=z.device)
+    w = torch.empty(t, top_k, dtype=torch.float32, device=z.device)
+    _lib.check(_lib.load().chadq_moe_route(z.data_ptr(), idx.data_ptr(), w.data_ptr(), t, e, top_k, int(renorm), _stream()),
+               "chadq_moe_route")
+    return idx, w
+
+
+_moe_ws = {}  # (device, bytes) -> workspace tensor, reused between calls
+
+
+def moe_ffn(x: torch.Tensor, logits: torch.Tensor, experts, *, top_k: int = 2, renorm: bool = True) -> torch.Tensor:
+    """SiLU-gated mixture of experts.  x bf16 [T,H], logits fp32 [T,E]; experts: sequence of (gate, up, down)
+    QWeightInt4G32 triples with gate/up [F,H] and down [H,F].  Returns bf16 [T,H]."""
+    lib = _lib.load()
+    x = _dev(x, "x", torch.bfloat16)
+    z = _dev(logits, "logits", torch.float32)
+    t, h = x.shape
+    e = len(experts)
+    if z.shape != (t, e):
+        raise ValueError("logits must be [%d,%d]" % (t, e))
+    f = experts[0][0].N
+    arr = (_lib.MoeExpertI4G32 * e)()
+    keep = []
+    for i, (g, u, d) in enumerate(experts):
+        if (g.N, g.K) != (f, h) or (u.N, u.K) != (f, h) or (d.N, d.K) != (h, f):
+            raise ValueError("expert %d: gate/up must be [%d,%d] and down [%d,%d]" % (i, f, h, h, f))
+        ts = [_dev(g.packed, "gate", torch.uint8), _dev(g.scale, "gate scale", torch.float16),
+              _dev(u.packed, "up", torch.uint8), _dev(u.scale, "up scale", torch.float16),
+              _dev(d.packed, "down", torch.uint8), _dev(d.scale, "down scale", torch.float16)]
+        keep.append(ts)
+        arr[i] = _lib.MoeExpertI4G32(*[v.data_ptr() for v in ts])
+    need = lib.chadq_moe_ffn_i4g32_workspace_bytes(t, h, f, e, top_k)
+    if need == 0:
+        raise ValueError("unsupported MoE sizes T=%d H=%d F=%d E=%d top_k=%d" % (t, h, f, e, top_k))
+    key = (x.device, need)
+    ws = _moe_ws.get(key)
+    if ws is None:
+        ws = _moe_ws[key] = torch.empty(need, dtype=torch.uint8, device=x.device)
+    y = torch.empty(t, h, dtype=torch.bfloat16, device=x.device)
+    _lib.check(lib.chadq_moe_ffn_i4g32(x.data_ptr(), z.data_ptr(), arr, y.data_ptr(), t, h, f, e, top_k, int(renorm),
+                                       ws.data_ptr(), need, _stream()), "chadq_moe_ffn_i4g32")
+    return y

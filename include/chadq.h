@@ -101,6 +101,37 @@ int chadq_gemm_i4g32_bf16(const uint16_t *x_bf16, const uint8_t *wp, const uint1
 int chadq_gemm_i8row_bf16(const uint16_t *x_bf16, const int8_t *w8, const float *scale, uint16_t *y_bf16, int M,
                           int N, int K, void *stream);
 
+/* ---- mixture-of-experts FFN (benchmark config 3) ---------------------------------------- */
+
+/*
+ * softmax over E experts per token, then the top_k experts by logit (lowest index wins ties).
+ * idx int32 [T,top_k], w fp32 [T,top_k] = their probabilities, divided by their sum if renorm != 0.
+ * E <= 16, top_k <= min(E, 8).
+ */
+int chadq_moe_route(const float *logits, int32_t *idx, float *w, int T, int E, int top_k, int renorm, void *stream);
+
+/* Device pointers of one expert's int4 group-32 weights: gate and up are [F,H], down is [H,F]. */
+typedef struct chadq_moe_expert_i4g32 {
+    const uint8_t *wg;
+    const uint16_t *sg;
+    const uint8_t *wu;
+    const uint16_t *su;
+    const uint8_t *wd;
+    const uint16_t *sd;
+} chadq_moe_expert_i4g32;
+
+/* Bytes of device workspace chadq_moe_ffn_i4g32 needs for these sizes (0 if the sizes are invalid). */
+size_t chadq_moe_ffn_i4g32_workspace_bytes(int T, int H, int F, int E, int top_k);
+
+/*
+ * y[t] = bf16( sum_j w[t,j] * Wd_e ( bf16( silu(Wg_e x_t) * (Wu_e x_t) ) ) ),  e = idx[t,j] from chadq_moe_route.
+ * x bf16 [T,H], logits fp32 [T,E], y bf16 [T,H].  `experts` is a HOST array of E structs holding device pointers.
+ * H % 32 == 0, F % 32 == 0.  Runs entirely on `stream`; no host synchronisation, nothing allocated.
+ */
+int chadq_moe_ffn_i4g32(const uint16_t *x_bf16, const float *logits, const chadq_moe_expert_i4g32 *experts,
+                        uint16_t *y_bf16, int T, int H, int F, int E, int top_k, int renorm, void *workspace,
+                        size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

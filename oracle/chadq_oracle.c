@@ -152,7 +152,7 @@ void oracle_moe_route(const float *logits, int32_t *idx, float *w, int T, int E,
                 for (int i = 0; i < j; ++i)
                     if (idx[(int64_t)t * top_k + i] == e) taken = 1;
                 if (taken) continue;
-                if (best < 0 || p[e] > p[best]) best = e;
+                if (best < 0 || z[e] > z[best]) best = e; /* order by logit: same set, no dependence on exp() rounding */
             }
             idx[(int64_t)t * top_k + j] = best;
             w[(int64_t)t * top_k + j] = p[best];

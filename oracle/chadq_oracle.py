@@ -154,7 +154,10 @@ def moe_route(logits: np.ndarray, top_k: int = 2, renorm: bool = True):
     Returns (idx int32 [T,top_k], w fp32 [T,top_k]).
     """
     p = softmax(logits)
-    idx = np.argsort(-p, axis=-1, kind="stable")[:, :top_k].astype(np.int32)
+    # softmax is monotonic, so the top_k probabilities belong to the top_k logits; ordering by the logits
+    # themselves keeps the choice independent of the last bit of exp() (a CPU and a GPU exp may differ there)
+    z = np.asarray(logits, dtype=np.float32)
+    idx = np.argsort(-z, axis=-1, kind="stable")[:, :top_k].astype(np.int32)
     w = np.take_along_axis(p, idx, axis=-1)
     if renorm:
         w = w / w.sum(axis=-1, keepdims=True)

@@ -260,3 +260,73 @@ def test_errors_surface_as_exceptions(ops):
     assert lib.chadq_gemv_i4g32(None, None, None, None, 1, 64, 100, None) == -2
     assert b"multiple of 32" in lib.chadq_last_error()
     assert lib.chadq_gemv_i4g32(None, None, None, None, 1, 0, 128, None) == 0  # empty output: nothing to do
+
+
+# ------------------------------------------------------------------ MoE (config 3)
+def _experts(seed, e, h, f):
+    """e experts of random int4 group-32 weights: numpy tuples for the oracle and device containers for the ops."""
+    from chadslab_amd import QWeightInt4G32
+
+    r = rng(seed)
+    host, dev = [], []
+    for _ in range(e):
+        hw, dw = [], []
+        for (n, k) in ((f, h), (f, h), (h, f)):
+            u = r.integers(0, 16, (n, k), dtype=np.uint8)
+            p = (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8)
+            s = (r.lognormal(-5, 0.5, (n, k // 32)) * (0.6 if n == h else 1.0)).astype(np.float16)
+            hw += [p, s]
+            dw.append(QWeightInt4G32(torch.from_numpy(p).to(DEV), torch.from_numpy(s).to(DEV)))
+        host.append(tuple(hw))
+        dev.append(tuple(dw))
+    return host, dev
+
+
+def test_moe_route_matches_oracle(ops):
+    r = rng(70)
+    logits = r.standard_normal((300, 8)).astype(np.float32)
+    logits[5, 2] = logits[5, 6] = logits[5].max() + 1.0   # tie for first place
+    logits[9, :] = 0.25                                    # all equal
+    logits[11, 1] = logits[11, 3]                          # tie somewhere
+    for top_k, renorm in ((2, True), (2, False), (1, True), (4, True)):
+        idx, w = ops.moe_route(torch.from_numpy(logits).to(DEV), top_k, renorm)
+        oi, ow = O.moe_route(logits, top_k, renorm)
+        assert np.array_equal(idx.cpu().numpy(), oi)       # indices bit-exact
+        assert np.allclose(w.cpu().numpy(), ow, rtol=2e-5, atol=1e-7)
+    assert idx.cpu().numpy()[9].tolist() == [0, 1, 2, 3]
+
+
+def test_moe_golden(ops):
+    from chadslab_amd import QWeightInt4G32
+
+    g = np.load(os.path.join(GOLD, "moe_t16_h64_f96_e4.npz"))
+    experts = [tuple(QWeightInt4G32(torch.from_numpy(g["e%d_%s_p" % (i, n)]).to(DEV), torch.from_numpy(g["e%d_%s_s" % (i, n)]).to(DEV))
+                     for n in "gud") for i in range(4)]
+    y = ops.moe_ffn(bf16_tensor(g["x_bf16"]), torch.from_numpy(g["logits"]).to(DEV), experts, top_k=2, renorm=True)
+    assert O.rel_l2(O.bf16_to_f32(bits(y)), O.bf16_to_f32(g["y_bf16"])) <= TOL_BF16
+
+
+@pytest.mark.parametrize("t,h,f,e,top_k", [(256, 512, 1024, 8, 2), (37, 128, 160, 3, 1), (64, 256, 256, 1, 1), (130, 256, 512, 16, 4)])
+def test_moe_ffn(ops, t, h, f, e, top_k):
+    host, dev = _experts(80 + t, e, h, f)
+    r = rng(81 + t)
+    xb = O.f32_to_bf16(r.standard_normal((t, h)).astype(np.float32))
+    logits = r.standard_normal((t, e)).astype(np.float32)
+    y = O.bf16_to_f32(bits(ops.moe_ffn(bf16_tensor(xb), torch.from_numpy(logits).to(DEV), dev, top_k=top_k, renorm=True)))
+    ref = O.bf16_to_f32(O.moe_qffn(xb, logits, host, top_k, True))
+    assert np.isfinite(y).all() and O.rel_l2(y, ref) <= TOL_BF16
+    # token order does not matter
+    perm = r.permutation(t)
+    yp = O.bf16_to_f32(bits(ops.moe_ffn(bf16_tensor(xb[perm]), torch.from_numpy(logits[perm]).to(DEV), dev, top_k=top_k, renorm=True)))
+    assert np.array_equal(yp, y[perm])
+
+
+def test_moe_config3_full_size(ops):
+    t, h, f, e = 256, 4096, 14336, 8
+    host, dev = _experts(1003, e, h, f)
+    r = rng(1003)
+    logits = r.standard_normal((t, e)).astype(np.float32)
+    xb = O.f32_to_bf16(r.standard_normal((t, h)).astype(np.float32))
+    y = O.bf16_to_f32(bits(ops.moe_ffn(bf16_tensor(xb), torch.from_numpy(logits).to(DEV), dev, top_k=2, renorm=True)))
+    ref = O.bf16_to_f32(O.moe_qffn(xb, logits, host, 2, True))
+    assert O.rel_l2(y, ref) <= TOL_BF16
