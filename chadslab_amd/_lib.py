@@ -6,7 +6,7 @@ There is no CPU or PyTorch fallback.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libchadq.so"
@@ -28,6 +28,14 @@ SIGNATURES = {
     "chadq_moe_ffn_i4g32_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "chadq_moe_ffn_i4g32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_void_p, c_size_t, c_void_p]),
+    "chadq_embed_i4g32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "chadq_add_rmsnorm_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p]),
+    "chadq_rope_kv_write": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float,
+                                    c_void_p]),
+    "chadq_attn_decode_mqa_workspace_floats": (c_size_t, [c_int, c_int, c_int]),
+    "chadq_attn_decode_mqa": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "chadq_geglu_bf16": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
+    "chadq_argmax_f32": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
 }
 
 

@@ -56,6 +56,14 @@ int moe_route_launch(const float *, int32_t *, float *, int, int, int, int, hipS
 int moe_ffn_i4g32_launch(const uint16_t *, const float *, const chadq_moe_expert_i4g32 *, uint16_t *, int, int, int, int, int,
                          int, void *, hipStream_t);
 
+int embed_launch(const int32_t *, const uint8_t *, const uint16_t *, float *, int, int, hipStream_t);
+int add_rmsnorm_launch(float *, const float *, const float *, uint16_t *, int, float, hipStream_t);
+int rope_kv_launch(const float *, const int32_t *, float *, uint16_t *, uint16_t *, int, int, int, float, hipStream_t);
+int attn_mqa_launch(const float *, const uint16_t *, const uint16_t *, const int32_t *, float *, uint16_t *, int, int, int,
+                    hipStream_t);
+int geglu_launch(const float *, uint16_t *, int, hipStream_t);
+int argmax_launch(const float *, int, float *, int32_t *, int32_t *, int32_t *, int, hipStream_t);
+
 }  // namespace chadq
 
 using namespace chadq;
@@ -189,6 +197,63 @@ int chadq_moe_ffn_i4g32(const uint16_t *x_bf16, const float *logits, const chadq
     CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(workspace) && aligned16(y_bf16), CHADQ_ERR_ALIGN,
                   "chadq_moe_ffn_i4g32: x, y and workspace must be 16-byte aligned");
     return moe_ffn_i4g32_launch(x_bf16, logits, experts, y_bf16, T, H, F, E, top_k, renorm, workspace, st);
+}
+
+int chadq_embed_i4g32(const int32_t *token, const uint8_t *wp, const uint16_t *scale_f16, float *x, int d, int V, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(d >= 32 && d % 32 == 0 && V >= 1, CHADQ_ERR_SHAPE,
+                  "chadq_embed_i4g32: d=%d must be a positive multiple of 32, V=%d positive", d, V);
+    CHADQ_REQUIRE(token && wp && scale_f16 && x, CHADQ_ERR_NULL, "chadq_embed_i4g32: null pointer");
+    return embed_launch(token, wp, scale_f16, x, d, V, st);
+}
+
+int chadq_add_rmsnorm_bf16(float *res, const float *delta, const float *w, uint16_t *y_bf16, int d, float eps,
+                           void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(d >= 1, CHADQ_ERR_SHAPE, "chadq_add_rmsnorm_bf16: d=%d", d);
+    CHADQ_REQUIRE(res && w && y_bf16, CHADQ_ERR_NULL, "chadq_add_rmsnorm_bf16: null pointer");
+    return add_rmsnorm_launch(res, delta, w, y_bf16, d, eps, st);
+}
+
+int chadq_rope_kv_write(const float *qkv, const int32_t *pos, float *q_out, uint16_t *kcache_bf16,
+                        uint16_t *vcache_bf16, int hq, int dh, int max_ctx, float base, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(hq >= 1 && dh >= 2 && dh % 2 == 0 && max_ctx >= 1, CHADQ_ERR_SHAPE,
+                  "chadq_rope_kv_write: hq=%d dh=%d max_ctx=%d", hq, dh, max_ctx);
+    CHADQ_REQUIRE(qkv && pos && q_out && kcache_bf16 && vcache_bf16, CHADQ_ERR_NULL, "chadq_rope_kv_write: null pointer");
+    return rope_kv_launch(qkv, pos, q_out, kcache_bf16, vcache_bf16, hq, dh, max_ctx, base, st);
+}
+
+size_t chadq_attn_decode_mqa_workspace_floats(int hq, int dh, int max_ctx) {
+    if (hq < 1 || dh < 1 || max_ctx < 1) return 0;
+    return (size_t)((max_ctx + 63) / 64) * hq * (dh + 2);
+}
+
+int chadq_attn_decode_mqa(const float *q, const uint16_t *kcache_bf16, const uint16_t *vcache_bf16, const int32_t *pos,
+                          float *workspace, uint16_t *out_bf16, int hq, int dh, int max_ctx, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(hq >= 1 && hq <= 8 && dh >= 8 && dh <= 256 && dh % 8 == 0 && max_ctx >= 1, CHADQ_ERR_SHAPE,
+                  "chadq_attn_decode_mqa: hq=%d dh=%d max_ctx=%d (hq <= 8, dh <= 256 and a multiple of 8)", hq, dh, max_ctx);
+    CHADQ_REQUIRE(q && kcache_bf16 && vcache_bf16 && pos && workspace && out_bf16, CHADQ_ERR_NULL,
+                  "chadq_attn_decode_mqa: null pointer");
+    CHADQ_REQUIRE(aligned16(kcache_bf16), CHADQ_ERR_ALIGN, "chadq_attn_decode_mqa: kcache must be 16-byte aligned");
+    return attn_mqa_launch(q, kcache_bf16, vcache_bf16, pos, workspace, out_bf16, hq, dh, max_ctx, st);
+}
+
+int chadq_geglu_bf16(const float *gu, uint16_t *h_bf16, int F, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(F >= 1, CHADQ_ERR_SHAPE, "chadq_geglu_bf16: F=%d", F);
+    CHADQ_REQUIRE(gu && h_bf16, CHADQ_ERR_NULL, "chadq_geglu_bf16: null pointer");
+    return geglu_launch(gu, h_bf16, F, st);
+}
+
+int chadq_argmax_f32(const float *v, int n, void *scratch, int32_t *token, int32_t *pos, int advance, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(n >= 1, CHADQ_ERR_SHAPE, "chadq_argmax_f32: n=%d", n);
+    CHADQ_REQUIRE(v && scratch && token && (pos || !advance), CHADQ_ERR_NULL, "chadq_argmax_f32: null pointer");
+    float *pv = reinterpret_cast<float *>(scratch);
+    int32_t *pi = reinterpret_cast<int32_t *>(pv + 256);
+    return argmax_launch(v, n, pv, pi, token, pos, advance, st);
 }
 
 }  // extern "C"

@@ -37,10 +37,10 @@
 
 namespace chadq {
 
-constexpr int KC = 4096;  // k per chunk
 constexpr int ZERO_BYTES = 1024;
 
-template <int MT, int HP, int S, int RBW>
+// KC = k per chunk (4096, or 2048 for short rows)
+template <int MT, int HP, int S, int RBW, int KC>
 struct GemvCfg {
     static constexpr int P = 16 / HP;                    // weight rows per MFMA tile
     static constexpr int MPASS = 4 / HP;                 // activation rows per pass
@@ -65,11 +65,11 @@ struct GemvCfg {
 };
 
 // waves_per_eu(4): at most 128 VGPRs, which also makes the compiler pick the MFMA form that writes VGPRs.
-template <int MT, int HP, int S, int RBW, int D>
+template <int MT, int HP, int S, int RBW, int D, int KC>
 __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) void gemv_i4g32_mfma_kernel(
     const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
     float *__restrict__ y, int N, int K) {
-    typedef GemvCfg<MT, HP, S, RBW> C;
+    typedef GemvCfg<MT, HP, S, RBW, KC> C;
     constexpr int M = MT, MP = C::MP, MPASS = C::MPASS, P = C::P, KS = C::KS, T = C::T, XI = C::XI;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -238,18 +238,18 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
 
 int gemv_i4g32_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
 
-template <int MT, int HP, int S, int RBW, int D = 8>
+template <int MT, int HP, int S, int RBW, int D, int KC = 4096>
 static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K,
                        hipStream_t st) {
-    typedef GemvCfg<MT, HP, S, RBW> C;
+    typedef GemvCfg<MT, HP, S, RBW, KC> C;
     static bool attr_set = false;
     if (!attr_set) {
-        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D>),
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::TOTAL));
         attr_set = true;
     }
     const int units = (N + C::UR - 1) / C::UR;
-    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D>), dim3((units + RBW - 1) / RBW), dim3(256 * RBW), C::TOTAL,
+    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC>), dim3((units + RBW - 1) / RBW), dim3(256 * RBW), C::TOTAL,
                        st, x, wp, sc, y, N, K);
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma launch");
 }
@@ -267,7 +267,11 @@ int gemv_i4g32_mfma_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_
         int rc = 0;
         // <rows, K-parts, steps per wave, 4-wave groups per workgroup, prefetch distance>, picked by measurement
         switch (mm) {
-            case 1: rc = launch_mfma<1, 4, 8, 1, 3>(xm, wp, sc, ym, N, K, st); break;
+            case 1:
+                // rows of at most 2048 k: 2048-wide chunks, 4 steps per wave (no loads past the row)
+                rc = K <= 2048 ? launch_mfma<1, 4, 4, 1, 4, 2048>(xm, wp, sc, ym, N, K, st)
+                               : launch_mfma<1, 4, 8, 1, 3>(xm, wp, sc, ym, N, K, st);
+                break;
             case 2: rc = launch_mfma<2, 2, 8, 1, 2>(xm, wp, sc, ym, N, K, st); break;
             case 3: rc = launch_mfma<3, 1, 8, 1, 8>(xm, wp, sc, ym, N, K, st); break;
             case 4: rc = launch_mfma<4, 1, 8, 1, 8>(xm, wp, sc, ym, N, K, st); break;

@@ -1,0 +1,150 @@
+"""A Gemma-2B-shaped decoder-only transformer step (batch 1) on int4 group-32 weights, built from the library's
+GEMV and the small decode kernels.  Every launch goes through the C ABI on torch's current stream; position
+and token live in device memory, so the whole step can be captured once in a HIP graph and replayed.
+
+Model conventions are this build's plain choices (the benchmark text fixes shapes only): RMSNorm y = x/rms*w,
+rotate-half RoPE base 10000, multi-query attention with one KV head, GeGLU with tanh-GELU, tied int4
+embedding / output table without embedding scaling or logit soft-capping.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List
+
+import torch
+
+from . import _lib
+from .formats import QWeightInt4G32, quantize_int4_g32
+
+
+@dataclass
+class DecoderConfig:
+    n_layers: int = 18
+    d: int = 2048
+    hq: int = 8
+    dh: int = 256
+    ffn: int = 16384
+    vocab: int = 256000
+    max_ctx: int = 4096
+    eps: float = 1e-6
+    rope_base: float = 10000.0
+
+
+def random_weights(cfg: DecoderConfig, seed: int, device) -> Dict:
+    """Random-init fp32 weights ~N(0, 0.02) quantised to int4 group-32 (absmax/7 per group); norms ~1."""
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+
+    def q(n, k):
+        # generate and quantise in slabs to bound memory (the output table is 2 GB in fp32)
+        packed, scale = [], []
+        for r0 in range(0, n, 32768):
+            w = torch.randn(min(32768, n - r0), k, device=device, generator=g) * 0.02
+            qw = quantize_int4_g32(w)
+            packed.append(qw.packed)
+            scale.append(qw.scale)
+        return QWeightInt4G32(torch.cat(packed), torch.cat(scale))
+
+    def norm():
+        return (1.0 + 0.1 * torch.randn(cfg.d, device=device, generator=g)).float()
+
+    layers = []
+    for _ in range(cfg.n_layers):
+        layers.append({
+            "ln1": norm(), "wqkv": q((cfg.hq + 2) * cfg.dh, cfg.d), "wo": q(cfg.d, cfg.hq * cfg.dh),
+            "ln2": norm(), "wgu": q(2 * cfg.ffn, cfg.d), "wd": q(cfg.d, cfg.ffn),
+        })
+    return {"layers": layers, "lnf": norm(), "emb": q(cfg.vocab, cfg.d)}
+
+
+class QuantDecoder:
+    def __init__(self, cfg: DecoderConfig, weights: Dict, device="cuda:0"):
+        if not torch.cuda.is_available():
+            raise RuntimeError("QuantDecoder needs the GPU (there is no CPU path)")
+        self.cfg, self.w, self.dev = cfg, weights, torch.device(device)
+        self.lib = _lib.load()
+        f32, bf16, i32 = torch.float32, torch.bfloat16, torch.int32
+        z = lambda n, dt: torch.zeros(n, dtype=dt, device=self.dev)  # noqa: E731
+        c = cfg
+        self.x, self.xn = z(c.d, f32), z(c.d, bf16)
+        self.qkv, self.q = z((c.hq + 2) * c.dh, f32), z(c.hq * c.dh, f32)
+        self.att, self.ao = z(c.hq * c.dh, bf16), z(c.d, f32)
+        self.gu, self.h, self.dn = z(2 * c.ffn, f32), z(c.ffn, bf16), z(c.d, f32)
+        self.logits = z(c.vocab, f32)
+        self.part = z(self.lib.chadq_attn_decode_mqa_workspace_floats(c.hq, c.dh, c.max_ctx), f32)
+        self.scratch = z(512, f32)
+        self.token, self.pos = z(1, i32), z(1, i32)
+        self.kcache = [z(c.max_ctx * c.dh, bf16) for _ in range(c.n_layers)]
+        self.vcache = [z(c.max_ctx * c.dh, bf16) for _ in range(c.n_layers)]
+        self.graph = None
+
+    # ---- single launches -------------------------------------------------------------------------------
+    def _s(self):
+        return torch.cuda.current_stream().cuda_stream
+
+    def _gemv(self, x_bf16, qw: QWeightInt4G32, y):
+        _lib.check(self.lib.chadq_gemv_i4g32(x_bf16.data_ptr(), qw.packed.data_ptr(), qw.scale.data_ptr(), y.data_ptr(),
+                                             1, qw.N, qw.K, self._s()), "chadq_gemv_i4g32")
+
+    def _norm(self, delta, w):
+        _lib.check(self.lib.chadq_add_rmsnorm_bf16(self.x.data_ptr(), delta.data_ptr() if delta is not None else None,
+                                                   w.data_ptr(), self.xn.data_ptr(), self.cfg.d, self.cfg.eps, self._s()),
+                   "chadq_add_rmsnorm_bf16")
+
+    def step(self) -> None:
+        """One token: reads token/pos from device memory, leaves the next token and pos+1 there."""
+        c, lib, s = self.cfg, self.lib, self._s()
+        _lib.check(lib.chadq_embed_i4g32(self.token.data_ptr(), self.w["emb"].packed.data_ptr(), self.w["emb"].scale.data_ptr(),
+                                         self.x.data_ptr(), c.d, c.vocab, s), "chadq_embed_i4g32")
+        pending = None
+        for li, L in enumerate(self.w["layers"]):
+            self._norm(pending, L["ln1"])
+            self._gemv(self.xn, L["wqkv"], self.qkv)
+            _lib.check(lib.chadq_rope_kv_write(self.qkv.data_ptr(), self.pos.data_ptr(), self.q.data_ptr(),
+                                               self.kcache[li].data_ptr(), self.vcache[li].data_ptr(), c.hq, c.dh,
+                                               c.max_ctx, c.rope_base, s), "chadq_rope_kv_write")
+            _lib.check(lib.chadq_attn_decode_mqa(self.q.data_ptr(), self.kcache[li].data_ptr(), self.vcache[li].data_ptr(),
+                                                 self.pos.data_ptr(), self.part.data_ptr(), self.att.data_ptr(), c.hq, c.dh,
+                                                 c.max_ctx, s), "chadq_attn_decode_mqa")
+            self._gemv(self.att, L["wo"], self.ao)
+            self._norm(self.ao, L["ln2"])
+            self._gemv(self.xn, L["wgu"], self.gu)
+            _lib.check(lib.chadq_geglu_bf16(self.gu.data_ptr(), self.h.data_ptr(), c.ffn, s), "chadq_geglu_bf16")
+            self._gemv(self.h, L["wd"], self.dn)
+            pending = self.dn
+        self._norm(pending, self.w["lnf"])
+        self._gemv(self.xn, self.w["emb"], self.logits)
+        _lib.check(lib.chadq_argmax_f32(self.logits.data_ptr(), c.vocab, self.scratch.data_ptr(), self.token.data_ptr(),
+                                        self.pos.data_ptr(), 1, s), "chadq_argmax_f32")
+
+    def capture(self) -> None:
+        """Captures step() in a HIP graph (after one eager warm-up step whose effects are undone)."""
+        tok, pos = self.token.clone(), self.pos.clone()
+        st = torch.cuda.Stream()
+        st.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(st):
+            self.step()
+            torch.cuda.synchronize()
+            self.token.copy_(tok)
+            self.pos.copy_(pos)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=st):
+                self.step()
+            self.token.copy_(tok)
+            self.pos.copy_(pos)
+        torch.cuda.current_stream().wait_stream(st)
+        torch.cuda.synchronize()
+        self.graph = g
+
+    def generate(self, first_token: int, pos: int, n: int) -> List[int]:
+        """Greedy decoding of n tokens starting from `first_token` at position `pos` (the cache holds pos rows)."""
+        self.token.fill_(first_token)
+        self.pos.fill_(pos)
+        out = []
+        for _ in range(n):
+            if self.graph is not None:
+                self.graph.replay()
+            else:
+                self.step()
+            out.append(int(self.token.item()))
+        return out

@@ -132,6 +132,44 @@ int chadq_moe_ffn_i4g32(const uint16_t *x_bf16, const float *logits, const chadq
                         uint16_t *y_bf16, int T, int H, int F, int E, int top_k, int renorm, void *workspace,
                         size_t workspace_bytes, void *stream);
 
+/* ---- decode-step pieces around the GEMVs (benchmark config 4), batch 1 ------------------- */
+/* The position and the current token live in device memory so that one captured HIP graph serves every step. */
+
+/* x[d] fp32 = dequantised row token[0] (clamped to [0,V-1]) of the tied int4 group-32 table [V,d]. */
+int chadq_embed_i4g32(const int32_t *token, const uint8_t *wp, const uint16_t *scale_f16, float *x, int d, int V,
+                      void *stream);
+
+/* res[d] += delta[d] (skipped if delta is NULL); y[d] = bf16( res / sqrt(mean(res^2) + eps) * w ). */
+int chadq_add_rmsnorm_bf16(float *res, const float *delta, const float *w, uint16_t *y_bf16, int d, float eps,
+                           void *stream);
+
+/*
+ * qkv fp32 = [hq*dh | dh | dh].  Rotate-half RoPE (given base) at position pos[0] on q and k; q_out fp32 [hq*dh];
+ * row pos[0] of the bf16 caches kcache/vcache [max_ctx,dh] receives k and v.  pos[0] is clamped to [0,max_ctx-1]
+ * here and in chadq_attn_decode_mqa, so a runaway position cannot address outside the cache.
+ */
+int chadq_rope_kv_write(const float *qkv, const int32_t *pos, float *q_out, uint16_t *kcache_bf16,
+                        uint16_t *vcache_bf16, int hq, int dh, int max_ctx, float base, void *stream);
+
+/* Floats of workspace chadq_attn_decode_mqa needs for a cache of max_ctx rows. */
+size_t chadq_attn_decode_mqa_workspace_floats(int hq, int dh, int max_ctx);
+
+/*
+ * Multi-query decode attention over cache rows 0..pos[0]: out bf16 [hq*dh] = softmax(q k^T / sqrt(dh)) v per head,
+ * all heads sharing one K/V.  hq <= 8, dh <= 256 and a multiple of 8.
+ */
+int chadq_attn_decode_mqa(const float *q, const uint16_t *kcache_bf16, const uint16_t *vcache_bf16, const int32_t *pos,
+                          float *workspace, uint16_t *out_bf16, int hq, int dh, int max_ctx, void *stream);
+
+/* h[F] = bf16( gelu_tanh(gu[i]) * gu[F+i] ). */
+int chadq_geglu_bf16(const float *gu, uint16_t *h_bf16, int F, void *stream);
+
+/*
+ * token[0] = argmax of v[0..n) (lowest index wins ties); pos[0] += 1 if advance != 0.
+ * scratch: 256 floats followed by 256 int32 (2048 bytes).
+ */
+int chadq_argmax_f32(const float *v, int n, void *scratch, int32_t *token, int32_t *pos, int advance, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

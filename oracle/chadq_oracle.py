@@ -220,3 +220,63 @@ def rel_l2(a: np.ndarray, ref: np.ndarray) -> float:
     ref = np.asarray(ref, dtype=np.float64)
     d = np.linalg.norm(ref)
     return float(np.linalg.norm(a - ref) / (d if d > 0 else 1.0))
+
+
+# --------------------------------------------------------------------------- decode step (config 4)
+# Conventions (this build's plain choices; the benchmark text fixes shapes only, so parity with the
+# reference is unpinned here): RMSNorm y = x / sqrt(mean(x^2) + eps) * w; rotate-half RoPE, base 10000;
+# multi-query attention (one KV head), scores / sqrt(dh), KV cache in bf16; GeGLU with tanh-GELU; tied int4
+# embedding / output table, no embedding scaling, no logit soft-cap; residual stream in fp32; every GEMV
+# input rounded to bf16 (that is what the kernels consume).
+def rmsnorm(x, w, eps):
+    x = np.asarray(x, dtype=np.float32)
+    return (x / np.sqrt(np.mean(x * x, dtype=np.float32) + np.float32(eps)) * np.asarray(w, dtype=np.float32)).astype(np.float32)
+
+
+def rope_rotate_half(v, pos, base=10000.0):
+    """v fp32 [..., dh]: pairs (j, j+dh/2) rotated by pos * base^(-2j/dh)."""
+    v = np.asarray(v, dtype=np.float32)
+    dh = v.shape[-1]
+    half = dh // 2
+    inv = np.power(np.float32(base), (-2.0 * np.arange(half, dtype=np.float32) / np.float32(dh)).astype(np.float32)).astype(np.float32)
+    ang = (np.float32(pos) * inv).astype(np.float32)
+    cs, sn = np.cos(ang.astype(np.float64)).astype(np.float32), np.sin(ang.astype(np.float64)).astype(np.float32)
+    a, b = v[..., :half], v[..., half:]
+    return np.concatenate([a * cs - b * sn, b * cs + a * sn], axis=-1).astype(np.float32)
+
+
+def gelu_tanh(x):
+    x = np.asarray(x, dtype=np.float32)
+    return (0.5 * x * (1.0 + np.tanh(np.float32(0.7978845608028654) * (x + np.float32(0.044715) * x * x * x)))).astype(np.float32)
+
+
+def decode_step(model, token, pos, kcache, vcache, hq, dh, eps=1e-6, base=10000.0):
+    """One token of a decoder-only transformer on int4 group-32 weights.  model: {"layers": [{"ln1","wqkv",
+    "wo","ln2","wgu","wd"}], "lnf", "emb"} with weights as (packed, scale) tuples.  kcache/vcache: per layer
+    bf16 bit arrays [max_ctx, dh], row `pos` is written.  Returns fp32 logits [V]."""
+    ep, es = model["emb"]
+    d = ep.shape[1] * 2
+    x = dequant_int4g32(ep[token:token + 1], es[token:token + 1])[0]
+    for li, L in enumerate(model["layers"]):
+        xn = f32_to_bf16(rmsnorm(x, L["ln1"], eps))[None, :]
+        qkv = qgemv_int4g32(xn, *L["wqkv"])[0]
+        q = rope_rotate_half(qkv[: hq * dh].reshape(hq, dh), pos, base)
+        k = rope_rotate_half(qkv[hq * dh: (hq + 1) * dh], pos, base)
+        v = qkv[(hq + 1) * dh:]
+        kcache[li][pos] = f32_to_bf16(k)
+        vcache[li][pos] = f32_to_bf16(v)
+        kk = bf16_to_f32(kcache[li][: pos + 1])
+        vv = bf16_to_f32(vcache[li][: pos + 1])
+        sc = (q @ kk.T) / np.float32(np.sqrt(dh))
+        sc = sc - sc.max(axis=-1, keepdims=True)
+        p = np.exp(sc)
+        p = p / p.sum(axis=-1, keepdims=True)
+        att = f32_to_bf16((p @ vv).astype(np.float32)).reshape(1, hq * dh)
+        x = x + qgemv_int4g32(att, *L["wo"])[0]
+        xn = f32_to_bf16(rmsnorm(x, L["ln2"], eps))[None, :]
+        gu = qgemv_int4g32(xn, *L["wgu"])[0]
+        f = gu.shape[0] // 2
+        h = f32_to_bf16(gelu_tanh(gu[:f]) * gu[f:])[None, :]
+        x = x + qgemv_int4g32(h, *L["wd"])[0]
+    xn = f32_to_bf16(rmsnorm(x, model["lnf"], eps))[None, :]
+    return qgemv_int4g32(xn, ep, es)[0]

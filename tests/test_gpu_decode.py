@@ -1,0 +1,254 @@
+"""GPU parity of the decode-step kernels (called through the C ABI) and of the whole decoder step against the
+CPU oracle on the same seeded inputs.  Tolerances: fp32 pieces rel-L2 <= 1e-3 (1e-5-ish in practice), bf16
+outputs <= 1e-2, logits of a whole step <= 1e-2 with the same greedy token.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import chadq_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from chadslab_amd import _lib
+
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return _lib.load()
+
+
+def chk(rc, what):
+    from chadslab_amd import _lib
+
+    _lib.check(rc, what)
+
+
+def bits(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def bf16_tensor(b):
+    return torch.from_numpy(np.ascontiguousarray(b).view(np.int16)).view(torch.bfloat16).to(DEV)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+@pytest.mark.parametrize("d", [32, 96, 2048, 3000])
+def test_add_rmsnorm(lib, d):
+    r = rng(d)
+    res = r.standard_normal(d).astype(np.float32) * 2
+    delta = r.standard_normal(d).astype(np.float32)
+    w = (1 + 0.1 * r.standard_normal(d)).astype(np.float32)
+    tr, td, tw = dev(res), dev(delta), dev(w)
+    y = torch.zeros(d, dtype=torch.bfloat16, device=DEV)
+    chk(lib.chadq_add_rmsnorm_bf16(tr.data_ptr(), td.data_ptr(), tw.data_ptr(), y.data_ptr(), d, 1e-6, stream()), "norm")
+    want_res = res + delta
+    assert np.array_equal(tr.cpu().numpy(), want_res)
+    want = O.rmsnorm(want_res, w, 1e-6)
+    assert O.rel_l2(O.bf16_to_f32(bits(y)), want) < 5e-3  # bf16 rounding of the output
+    # delta = NULL leaves the residual alone
+    tr2 = dev(res)
+    chk(lib.chadq_add_rmsnorm_bf16(tr2.data_ptr(), None, tw.data_ptr(), y.data_ptr(), d, 1e-6, stream()), "norm")
+    assert np.array_equal(tr2.cpu().numpy(), res)
+    assert O.rel_l2(O.bf16_to_f32(bits(y)), O.rmsnorm(res, w, 1e-6)) < 5e-3
+
+
+@pytest.mark.parametrize("hq,dh,pos", [(8, 256, 0), (8, 256, 2047), (4, 64, 100), (1, 8, 3)])
+def test_rope_kv_write(lib, hq, dh, pos):
+    r = rng(hq * 1000 + dh + pos)
+    ctx = pos + 5
+    qkv = r.standard_normal((hq + 2) * dh).astype(np.float32)
+    tq = dev(qkv)
+    tp = torch.tensor([pos], dtype=torch.int32, device=DEV)
+    q = torch.zeros(hq * dh, dtype=torch.float32, device=DEV)
+    kc = torch.zeros(ctx * dh, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros(ctx * dh, dtype=torch.bfloat16, device=DEV)
+    chk(lib.chadq_rope_kv_write(tq.data_ptr(), tp.data_ptr(), q.data_ptr(), kc.data_ptr(), vc.data_ptr(), hq, dh, ctx, 10000.0,
+                                stream()), "rope")
+    want_q = O.rope_rotate_half(qkv[: hq * dh].reshape(hq, dh), pos).reshape(-1)
+    want_k = O.rope_rotate_half(qkv[hq * dh: (hq + 1) * dh], pos)
+    # fp32 sin/cos of angles up to ~2000 rad: argument rounding alone gives ~1e-4 absolute
+    assert np.abs(q.cpu().numpy() - want_q).max() < 2e-3
+    kb, vb = bits(kc).reshape(ctx, dh), bits(vc).reshape(ctx, dh)
+    assert np.abs(O.bf16_to_f32(kb[pos]) - want_k).max() < 4e-2
+    assert np.array_equal(vb[pos], O.f32_to_bf16(qkv[(hq + 1) * dh:]))
+    untouched = np.ones(ctx, bool)
+    untouched[pos] = False
+    assert not kb[untouched].any() and not vb[untouched].any()
+
+
+def test_rope_position_is_clamped_to_the_cache(lib):
+    hq, dh, ctx = 2, 16, 4
+    tq = dev(rng(1).standard_normal((hq + 2) * dh).astype(np.float32))
+    tp = torch.tensor([1000], dtype=torch.int32, device=DEV)
+    q = torch.zeros(hq * dh, dtype=torch.float32, device=DEV)
+    guard = torch.zeros((ctx + 4) * dh, dtype=torch.bfloat16, device=DEV)  # 4 rows of canary behind the cache
+    vc = torch.zeros((ctx + 4) * dh, dtype=torch.bfloat16, device=DEV)
+    chk(lib.chadq_rope_kv_write(tq.data_ptr(), tp.data_ptr(), q.data_ptr(), guard.data_ptr(), vc.data_ptr(), hq, dh, ctx,
+                                10000.0, stream()), "rope")
+    torch.cuda.synchronize()
+    assert not bits(guard)[ctx * dh:].any() and not bits(vc)[ctx * dh:].any()
+    assert bits(vc)[(ctx - 1) * dh: ctx * dh].any()  # landed in the last row
+
+
+@pytest.mark.parametrize("hq,dh,pos,max_ctx", [(8, 256, 0, 64), (8, 256, 63, 64), (8, 256, 64, 4096), (8, 256, 2047, 4096),
+                                               (8, 256, 4095, 4096), (3, 64, 200, 300), (1, 8, 70, 128)])
+def test_attn_decode_mqa(lib, hq, dh, pos, max_ctx):
+    r = rng(hq + dh + pos)
+    q = r.standard_normal(hq * dh).astype(np.float32)
+    kc = O.f32_to_bf16(r.standard_normal((max_ctx, dh)).astype(np.float32))
+    vc = O.f32_to_bf16(r.standard_normal((max_ctx, dh)).astype(np.float32))
+    tq, tk, tv = dev(q), bf16_tensor(kc.reshape(-1)), bf16_tensor(vc.reshape(-1))
+    tp = torch.tensor([pos], dtype=torch.int32, device=DEV)
+    ws = torch.zeros(lib.chadq_attn_decode_mqa_workspace_floats(hq, dh, max_ctx), dtype=torch.float32, device=DEV)
+    out = torch.zeros(hq * dh, dtype=torch.bfloat16, device=DEV)
+    chk(lib.chadq_attn_decode_mqa(tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), tp.data_ptr(), ws.data_ptr(), out.data_ptr(),
+                                  hq, dh, max_ctx, stream()), "attn")
+    kk = O.bf16_to_f32(kc[: pos + 1]).astype(np.float64)
+    vv = O.bf16_to_f32(vc[: pos + 1]).astype(np.float64)
+    s = q.reshape(hq, dh).astype(np.float64) @ kk.T / np.sqrt(dh)
+    p = np.exp(s - s.max(-1, keepdims=True))
+    want = (p / p.sum(-1, keepdims=True)) @ vv
+    assert O.rel_l2(O.bf16_to_f32(bits(out)).reshape(hq, dh), want) < 1e-2
+
+
+@pytest.mark.parametrize("F", [1, 255, 16384])
+def test_geglu(lib, F):
+    gu = (rng(F).standard_normal(2 * F) * 3).astype(np.float32)
+    t = dev(gu)
+    h = torch.zeros(F, dtype=torch.bfloat16, device=DEV)
+    chk(lib.chadq_geglu_bf16(t.data_ptr(), h.data_ptr(), F, stream()), "geglu")
+    want = O.gelu_tanh(gu[:F]) * gu[F:]
+    assert O.rel_l2(O.bf16_to_f32(bits(h)), want) < 5e-3
+
+
+@pytest.mark.parametrize("n", [1, 7, 256, 70000, 256000])
+def test_argmax_and_advance(lib, n):
+    v = rng(n).standard_normal(n).astype(np.float32)
+    if n > 10:
+        v[[3, n - 2]] = v.max() + 1  # a tie: the lower index must win
+    t = dev(v)
+    scratch = torch.zeros(512, dtype=torch.float32, device=DEV)
+    tok = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    pos = torch.tensor([41], dtype=torch.int32, device=DEV)
+    chk(lib.chadq_argmax_f32(t.data_ptr(), n, scratch.data_ptr(), tok.data_ptr(), pos.data_ptr(), 1, stream()), "argmax")
+    assert int(tok.item()) == int(np.argmax(v)) and int(pos.item()) == 42
+    chk(lib.chadq_argmax_f32(t.data_ptr(), n, scratch.data_ptr(), tok.data_ptr(), None, 0, stream()), "argmax")
+    assert int(tok.item()) == int(np.argmax(v)) and int(pos.item()) == 42
+
+
+def test_embed_row(lib):
+    V, d = 50, 96
+    p, s = O.quantize_int4_g32(rng(9).standard_normal((V, d)).astype(np.float32))
+    tp_, ts = dev(p), dev(s)
+    x = torch.zeros(d, dtype=torch.float32, device=DEV)
+    for token in (0, 17, 49, 10 ** 6, -3):  # the last two are clamped into the table
+        tt = torch.tensor([token], dtype=torch.int32, device=DEV)
+        chk(lib.chadq_embed_i4g32(tt.data_ptr(), tp_.data_ptr(), ts.data_ptr(), x.data_ptr(), d, V, stream()), "embed")
+        row = min(max(token, 0), V - 1)
+        assert np.array_equal(x.cpu().numpy(), O.dequant_int4g32(p[row: row + 1], s[row: row + 1])[0])
+
+
+# ---------------------------------------------------------------------------------------------- whole step
+def _model(seed, cfg):
+    r = rng(seed)
+
+    def q(n, k):
+        return O.quantize_int4_g32((r.standard_normal((n, k)) * 0.05).astype(np.float32))
+
+    def norm():
+        return (1 + 0.1 * r.standard_normal(cfg.d)).astype(np.float32)
+
+    layers = [{"ln1": norm(), "wqkv": q((cfg.hq + 2) * cfg.dh, cfg.d), "wo": q(cfg.d, cfg.hq * cfg.dh), "ln2": norm(),
+               "wgu": q(2 * cfg.ffn, cfg.d), "wd": q(cfg.d, cfg.ffn)} for _ in range(cfg.n_layers)]
+    return {"layers": layers, "lnf": norm(), "emb": q(cfg.vocab, cfg.d)}
+
+
+def _upload(m):
+    from chadslab_amd import QWeightInt4G32
+
+    def qw(ps):
+        return QWeightInt4G32(dev(ps[0]), dev(ps[1]))
+
+    return {"layers": [{k: (qw(v) if isinstance(v, tuple) else dev(v)) for k, v in L.items()} for L in m["layers"]],
+            "lnf": dev(m["lnf"]), "emb": qw(m["emb"])}
+
+
+def _run_steps(cfg, seed, pos0, nsteps, use_graph):
+    from chadslab_amd.decoder import QuantDecoder
+
+    m = _model(seed, cfg)
+    dec = QuantDecoder(cfg, _upload(m), DEV)
+    r = rng(seed + 1)
+    kc = [O.f32_to_bf16(r.standard_normal((cfg.max_ctx, cfg.dh)).astype(np.float32)) for _ in range(cfg.n_layers)]
+    vc = [O.f32_to_bf16(r.standard_normal((cfg.max_ctx, cfg.dh)).astype(np.float32)) for _ in range(cfg.n_layers)]
+    for li in range(cfg.n_layers):
+        dec.kcache[li].copy_(bf16_tensor(kc[li].reshape(-1)))
+        dec.vcache[li].copy_(bf16_tensor(vc[li].reshape(-1)))
+    tok = 5
+    dec.token.fill_(tok)
+    dec.pos.fill_(pos0)
+    if use_graph:
+        dec.capture()
+    for step in range(nsteps):
+        want = O.decode_step(m, tok, pos0 + step, kc, vc, cfg.hq, cfg.dh, cfg.eps, cfg.rope_base)
+        if use_graph:
+            dec.graph.replay()
+        else:
+            dec.step()
+        torch.cuda.synchronize()
+        got = dec.logits.cpu().numpy()
+        assert O.rel_l2(got, want) < 1e-2, "step %d" % step
+        assert int(dec.pos.item()) == pos0 + step + 1
+        gtok = int(dec.token.item())
+        assert gtok == int(np.argmax(got))
+        # the greedy token must agree unless the oracle's top two logits are closer than the tolerance allows
+        top2 = np.sort(want)[-2:]
+        if top2[1] - top2[0] > 2e-2 * np.abs(want).max():
+            assert gtok == int(np.argmax(want)), "step %d" % step
+        # the caches must have received this step's row in every layer
+        for li in (0, cfg.n_layers - 1):
+            row = bits(dec.kcache[li]).reshape(cfg.max_ctx, cfg.dh)[pos0 + step]
+            assert O.rel_l2(O.bf16_to_f32(row), O.bf16_to_f32(kc[li][pos0 + step])) < 2e-2
+        tok = gtok
+        if gtok != int(np.argmax(want)):
+            break  # sequences diverge legitimately after a near-tie
+
+
+def test_decoder_step_small_eager():
+    from chadslab_amd.decoder import DecoderConfig
+
+    _run_steps(DecoderConfig(n_layers=2, d=512, hq=4, dh=64, ffn=1024, vocab=1000, max_ctx=256), 40, 100, 4, False)
+
+
+def test_decoder_step_small_graph_replay():
+    from chadslab_amd.decoder import DecoderConfig
+
+    _run_steps(DecoderConfig(n_layers=2, d=512, hq=4, dh=64, ffn=1024, vocab=1000, max_ctx=256), 41, 60, 5, True)
+
+
+def test_decoder_step_odd_sizes_generic_gemv():
+    from chadslab_amd.decoder import DecoderConfig
+
+    # d and ffn that are not multiples of 256 send every GEMV down the generic kernel
+    _run_steps(DecoderConfig(n_layers=1, d=96, hq=2, dh=32, ffn=160, vocab=77, max_ctx=80), 42, 70, 3, False)
+
+
+def test_decoder_step_gemma_shapes_two_layers():
+    from chadslab_amd.decoder import DecoderConfig
+
+    # the benchmark's layer shapes (d 2048, 8 query heads x 256, 1 KV head, FFN 16384) at context 2048
+    _run_steps(DecoderConfig(n_layers=2, d=2048, hq=8, dh=256, ffn=16384, vocab=8192, max_ctx=2304), 43, 2047, 2, True)

@@ -330,3 +330,85 @@ def test_golden_fixtures_reproduce():
     assert np.array_equal(idx, gm["idx"]) and np.array_equal(w, gm["w"])
     experts = [tuple(gm["e%d_%s_%s" % (i, n, t)] for n in "gud" for t in "ps") for i in range(4)]
     assert np.array_equal(O.moe_qffn(gm["x_bf16"], gm["logits"], experts, 2, True), gm["y_bf16"])
+
+
+# ------------------------------------------------------------------ decode step
+def _tiny_model(seed, n_layers, d, hq, dh, ffn, vocab):
+    r = rng(seed)
+
+    def q(n, k):
+        return O.quantize_int4_g32((r.standard_normal((n, k)) * 0.05).astype(np.float32))
+
+    layers = [{"ln1": (1 + 0.1 * r.standard_normal(d)).astype(np.float32), "wqkv": q((hq + 2) * dh, d), "wo": q(d, hq * dh),
+               "ln2": (1 + 0.1 * r.standard_normal(d)).astype(np.float32), "wgu": q(2 * ffn, d), "wd": q(d, ffn)}
+              for _ in range(n_layers)]
+    return {"layers": layers, "lnf": (1 + 0.1 * r.standard_normal(d)).astype(np.float32), "emb": q(vocab, d)}
+
+
+def test_decode_pieces_against_torch():
+    r = rng(30)
+    x = r.standard_normal(96).astype(np.float32) * 3
+    w = r.standard_normal(96).astype(np.float32)
+    t = torch.from_numpy(x)
+    ref = t * torch.rsqrt(t.pow(2).mean() + 1e-6) * torch.from_numpy(w)
+    assert np.allclose(O.rmsnorm(x, w, 1e-6), ref.numpy(), rtol=1e-5, atol=1e-6)
+    g = r.standard_normal(1000).astype(np.float32) * 3
+    assert np.allclose(O.gelu_tanh(g), torch.nn.functional.gelu(torch.from_numpy(g), approximate="tanh").numpy(), rtol=1e-5, atol=1e-6)
+    # rotate-half RoPE as a complex rotation of (v[j], v[j+half])
+    v = r.standard_normal((3, 64)).astype(np.float32)
+    pos, half = 77, 32
+    ang = pos * (10000.0 ** (-2.0 * np.arange(half) / 64))
+    z = (v[:, :half] + 1j * v[:, half:]) * np.exp(1j * ang)
+    assert np.allclose(O.rope_rotate_half(v, pos), np.concatenate([z.real, z.imag], -1), rtol=1e-4, atol=1e-4)
+    assert np.allclose(O.rope_rotate_half(v, 0), v)  # position 0 is the identity
+    assert np.allclose(np.linalg.norm(O.rope_rotate_half(v, 1234), axis=-1), np.linalg.norm(v, axis=-1), rtol=1e-5)
+
+
+def test_decode_step_against_independent_torch_model():
+    n_layers, d, hq, dh, ffn, vocab, ctx = 2, 128, 2, 32, 256, 300, 40
+    m = _tiny_model(31, n_layers, d, hq, dh, ffn, vocab)
+    r = rng(32)
+    pos0 = 17
+    kc = [O.f32_to_bf16(r.standard_normal((ctx, dh)).astype(np.float32)) for _ in range(n_layers)]
+    vc = [O.f32_to_bf16(r.standard_normal((ctx, dh)).astype(np.float32)) for _ in range(n_layers)]
+    kc_t = [torch.from_numpy(O.bf16_to_f32(a).copy()) for a in kc]
+    vc_t = [torch.from_numpy(O.bf16_to_f32(a).copy()) for a in vc]
+
+    def bf(t):  # round a torch fp32 tensor to bf16 and back
+        return t.to(torch.bfloat16).to(torch.float32)
+
+    def deq(pw):
+        return torch.from_numpy(O.dequant_int4g32(*pw))
+
+    def torch_step(token, pos):
+        x = deq(m["emb"])[token].clone()
+        for li, L in enumerate(m["layers"]):
+            xn = bf(x * torch.rsqrt(x.pow(2).mean() + 1e-6) * torch.from_numpy(L["ln1"]))
+            qkv = deq(L["wqkv"]) @ xn
+            inv = 10000.0 ** (-2.0 * torch.arange(dh // 2, dtype=torch.float64) / dh)
+            rot = torch.polar(torch.ones(dh // 2, dtype=torch.float64), pos * inv)
+
+            def rope(vv):
+                zc = torch.complex(vv[..., : dh // 2].double(), vv[..., dh // 2:].double()) * rot
+                return torch.cat([zc.real, zc.imag], -1).float()
+
+            q = rope(qkv[: hq * dh].reshape(hq, dh))
+            kc_t[li][pos] = bf(rope(qkv[hq * dh: (hq + 1) * dh]))
+            vc_t[li][pos] = bf(qkv[(hq + 1) * dh:])
+            p = torch.softmax(q @ kc_t[li][: pos + 1].T / dh ** 0.5, dim=-1)
+            att = bf((p @ vc_t[li][: pos + 1]).reshape(-1))
+            x = x + deq(L["wo"]) @ att
+            xn = bf(x * torch.rsqrt(x.pow(2).mean() + 1e-6) * torch.from_numpy(L["ln2"]))
+            gu = deq(L["wgu"]) @ xn
+            h = bf(torch.nn.functional.gelu(gu[:ffn], approximate="tanh") * gu[ffn:])
+            x = x + deq(L["wd"]) @ h
+        xn = bf(x * torch.rsqrt(x.pow(2).mean() + 1e-6) * torch.from_numpy(m["lnf"]))
+        return (deq(m["emb"]) @ xn).numpy()
+
+    tok = 5
+    for step in range(3):
+        lo = O.decode_step(m, tok, pos0 + step, kc, vc, hq, dh)
+        lt = torch_step(tok, pos0 + step)
+        assert O.rel_l2(lo, lt) < 2e-3  # both round through bf16 at the same places; fp32 summation orders differ
+        assert int(lo.argmax()) == int(lt.argmax())
+        tok = int(lo.argmax())
