@@ -21,6 +21,7 @@ SIGNATURES = {
     "chadq_dequant_i4g32": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "chadq_dequant_i8row": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "chadq_gemv_i4g32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "chadq_gemv_i4g32_splitk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "chadq_gemv_i8row": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "chadq_gemm_i4g32_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "chadq_gemm_i8row_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
@@ -29,7 +30,7 @@ SIGNATURES = {
     "chadq_moe_ffn_i4g32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_void_p, c_size_t, c_void_p]),
     "chadq_embed_i4g32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
-    "chadq_add_rmsnorm_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p]),
+    "chadq_add_rmsnorm_bf16": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p]),
     "chadq_rope_kv_write": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float,
                                     c_void_p]),
     "chadq_attn_decode_mqa_workspace_floats": (c_size_t, [c_int, c_int, c_int]),

@@ -57,7 +57,8 @@ int moe_ffn_i4g32_launch(const uint16_t *, const float *, const chadq_moe_expert
                          int, void *, hipStream_t);
 
 int embed_launch(const int32_t *, const uint8_t *, const uint16_t *, float *, int, int, hipStream_t);
-int add_rmsnorm_launch(float *, const float *, const float *, uint16_t *, int, float, hipStream_t);
+int add_rmsnorm_launch(float *, const float *, int, const float *, uint16_t *, int, float, hipStream_t);
+int gemv_i4g32_splitk_launch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
 int rope_kv_launch(const float *, const int32_t *, float *, uint16_t *, uint16_t *, int, int, int, float, hipStream_t);
 int attn_mqa_launch(const float *, const uint16_t *, const uint16_t *, const int32_t *, float *, uint16_t *, int, int, int,
                     hipStream_t);
@@ -125,9 +126,20 @@ int chadq_gemv_i4g32(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *
     if (N == 0) return 0;
     CHADQ_REQUIRE(x_bf16 && wp && scale_f16 && y, CHADQ_ERR_NULL, "chadq_gemv_i4g32: null pointer");
     CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(wp), CHADQ_ERR_ALIGN, "chadq_gemv_i4g32: x and wp must be 16-byte aligned");
-    static const bool use_dot2 = getenv("CHADQ_GEMV_DOT2") != nullptr;  // development switch
-    if (use_dot2) return gemv_i4g32_dispatch(x_bf16, wp, scale_f16, y, M, N, K, st);
     return gemv_i4g32_mfma_dispatch(x_bf16, wp, scale_f16, y, M, N, K, st);
+}
+
+int chadq_gemv_i4g32_splitk(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *scale_f16, float *y_parts, int N,
+                            int K, int ksplit, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(N >= 1 && K >= 4096 && ksplit >= 1 && ksplit <= 64 && K % (ksplit * 4096) == 0, CHADQ_ERR_SHAPE,
+                  "chadq_gemv_i4g32_splitk: N=%d K=%d ksplit=%d (K must be a multiple of ksplit*4096)", N, K, ksplit);
+    CHADQ_REQUIRE((int64_t)N * (K / 2) < ((int64_t)1 << 31), CHADQ_ERR_SHAPE,
+                  "chadq_gemv_i4g32_splitk: N*K/2 = %lld bytes exceeds 2^31", (long long)N * (K / 2));
+    CHADQ_REQUIRE(x_bf16 && wp && scale_f16 && y_parts, CHADQ_ERR_NULL, "chadq_gemv_i4g32_splitk: null pointer");
+    CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(wp) && aligned16(scale_f16), CHADQ_ERR_ALIGN,
+                  "chadq_gemv_i4g32_splitk: x, wp and scale must be 16-byte aligned");
+    return gemv_i4g32_splitk_launch(x_bf16, wp, scale_f16, y_parts, N, K, ksplit, st);
 }
 
 int chadq_gemv_i8row(const float *x, const int8_t *w8, const float *scale, float *y, int M, int N, int K,
@@ -207,12 +219,12 @@ int chadq_embed_i4g32(const int32_t *token, const uint8_t *wp, const uint16_t *s
     return embed_launch(token, wp, scale_f16, x, d, V, st);
 }
 
-int chadq_add_rmsnorm_bf16(float *res, const float *delta, const float *w, uint16_t *y_bf16, int d, float eps,
+int chadq_add_rmsnorm_bf16(float *res, const float *delta, int n_delta, const float *w, uint16_t *y_bf16, int d, float eps,
                            void *stream) {
     ENTER();
-    CHADQ_REQUIRE(d >= 1, CHADQ_ERR_SHAPE, "chadq_add_rmsnorm_bf16: d=%d", d);
-    CHADQ_REQUIRE(res && w && y_bf16, CHADQ_ERR_NULL, "chadq_add_rmsnorm_bf16: null pointer");
-    return add_rmsnorm_launch(res, delta, w, y_bf16, d, eps, st);
+    CHADQ_REQUIRE(d >= 1 && n_delta >= 0 && n_delta <= 64, CHADQ_ERR_SHAPE, "chadq_add_rmsnorm_bf16: d=%d n_delta=%d", d, n_delta);
+    CHADQ_REQUIRE(res && w && y_bf16 && (delta || n_delta == 0), CHADQ_ERR_NULL, "chadq_add_rmsnorm_bf16: null pointer");
+    return add_rmsnorm_launch(res, delta, delta ? n_delta : 0, w, y_bf16, d, eps, st);
 }
 
 int chadq_rope_kv_write(const float *qkv, const int32_t *pos, float *q_out, uint16_t *kcache_bf16,
@@ -226,17 +238,20 @@ int chadq_rope_kv_write(const float *qkv, const int32_t *pos, float *q_out, uint
 
 size_t chadq_attn_decode_mqa_workspace_floats(int hq, int dh, int max_ctx) {
     if (hq < 1 || dh < 1 || max_ctx < 1) return 0;
-    return (size_t)((max_ctx + 63) / 64) * hq * (dh + 2);
+    return (size_t)((max_ctx + 31) / 32) * hq * (dh + 2);
 }
 
 int chadq_attn_decode_mqa(const float *q, const uint16_t *kcache_bf16, const uint16_t *vcache_bf16, const int32_t *pos,
                           float *workspace, uint16_t *out_bf16, int hq, int dh, int max_ctx, void *stream) {
     ENTER();
-    CHADQ_REQUIRE(hq >= 1 && hq <= 8 && dh >= 8 && dh <= 256 && dh % 8 == 0 && max_ctx >= 1, CHADQ_ERR_SHAPE,
-                  "chadq_attn_decode_mqa: hq=%d dh=%d max_ctx=%d (hq <= 8, dh <= 256 and a multiple of 8)", hq, dh, max_ctx);
+    CHADQ_REQUIRE(hq >= 1 && hq <= 8 && dh >= 8 && dh <= 256 && dh % 8 == 0 && max_ctx >= 1 && max_ctx <= 65536,
+                  CHADQ_ERR_SHAPE,
+                  "chadq_attn_decode_mqa: hq=%d dh=%d max_ctx=%d (hq <= 8, dh <= 256 and a multiple of 8, max_ctx <= 65536)", hq,
+                  dh, max_ctx);
     CHADQ_REQUIRE(q && kcache_bf16 && vcache_bf16 && pos && workspace && out_bf16, CHADQ_ERR_NULL,
                   "chadq_attn_decode_mqa: null pointer");
-    CHADQ_REQUIRE(aligned16(kcache_bf16), CHADQ_ERR_ALIGN, "chadq_attn_decode_mqa: kcache must be 16-byte aligned");
+    CHADQ_REQUIRE(aligned16(kcache_bf16) && aligned16(q), CHADQ_ERR_ALIGN,
+                  "chadq_attn_decode_mqa: q and kcache must be 16-byte aligned");
     return attn_mqa_launch(q, kcache_bf16, vcache_bf16, pos, workspace, out_bf16, hq, dh, max_ctx, st);
 }
 

@@ -10,8 +10,9 @@
 
 namespace chadq {
 
+// Sum / max over a workgroup of up to 256 threads; `scratch` holds one float per wave.  Both end with every
+// thread holding the result and may be called back to back on the same scratch.
 __device__ __forceinline__ float block_sum(float v, float *scratch) {
-    // 256 threads: wave sums, then 4 partials through LDS
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     __syncthreads();
@@ -19,6 +20,17 @@ __device__ __forceinline__ float block_sum(float v, float *scratch) {
     __syncthreads();
     float t = 0.f;
     for (int i = 0; i < (int)(blockDim.x >> 6); ++i) t += scratch[i];
+    return t;
+}
+
+__device__ __forceinline__ float block_max(float v, float *scratch) {
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = -INFINITY;
+    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) t = fmaxf(t, scratch[i]);
     return t;
 }
 
@@ -35,23 +47,63 @@ __global__ __launch_bounds__(256) void embed_i4g32_kernel(const int32_t *__restr
     }
 }
 
-// res += delta (if delta), y = bf16(rmsnorm(res) * w); one workgroup
-__global__ __launch_bounds__(256) void add_rmsnorm_kernel(float *__restrict__ res, const float *__restrict__ delta,
+// res += sum_j delta[j] (nd vectors of d floats, added in order), y = bf16(rmsnorm(res) * w); one workgroup.
+// Any d, any nd: the plain loop form.
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(float *__restrict__ res, const float *__restrict__ delta, int nd,
                                                           const float *__restrict__ w, uint16_t *__restrict__ y, int d,
                                                           float eps) {
     __shared__ float scratch[4];
     float ss = 0.f;
     for (int k = threadIdx.x; k < d; k += blockDim.x) {
         float v = res[k];
-        if (delta) {
-            v += delta[k];
-            res[k] = v;
-        }
+        for (int j = 0; j < nd; ++j) v += delta[(size_t)j * d + k];
+        if (nd > 0) res[k] = v;
         ss += v * v;
     }
     const float tot = block_sum(ss, scratch);
     const float r = rsqrtf(tot / (float)d + eps);
     for (int k = threadIdx.x; k < d; k += blockDim.x) y[k] = (uint16_t)f32_to_bf16_bits(res[k] * r * w[k]);
+}
+
+// The same for d % 4 == 0, d <= 1024 * NV: every load of the kernel is issued before anything waits (one memory
+// round trip instead of three), the vector stays in registers between the two passes.
+template <int NV, int ND>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float *__restrict__ res, const float *__restrict__ delta,
+                                                              const float *__restrict__ w, uint16_t *__restrict__ y, int d,
+                                                              float eps) {
+    __shared__ float scratch[4];
+    const int nv = d >> 2, tid = threadIdx.x;
+    f32x4 r[NV], wv[NV], dl[ND > 0 ? ND : 1][NV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int i = tid + 256 * j, ii = i < nv ? i : 0;  // clamped address, the data is discarded
+        r[j] = reinterpret_cast<const f32x4 *>(res)[ii];
+        wv[j] = reinterpret_cast<const f32x4 *>(w)[ii];
+#pragma unroll
+        for (int s = 0; s < ND; ++s) dl[s][j] = reinterpret_cast<const f32x4 *>(delta)[(size_t)s * nv + ii];
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int i = tid + 256 * j;
+#pragma unroll
+        for (int s = 0; s < ND; ++s) r[j] += dl[s][j];
+        if (i < nv) {
+            if (ND > 0) reinterpret_cast<f32x4 *>(res)[i] = r[j];
+            ss += r[j].x * r[j].x + r[j].y * r[j].y + r[j].z * r[j].z + r[j].w * r[j].w;
+        }
+    }
+    const float tot = block_sum(ss, scratch);
+    const float rinv = rsqrtf(tot / (float)d + eps);
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int i = tid + 256 * j;
+        if (i < nv) {
+            const uint32_t lo = f32_to_bf16_bits(r[j].x * rinv * wv[j].x) | (f32_to_bf16_bits(r[j].y * rinv * wv[j].y) << 16);
+            const uint32_t hi = f32_to_bf16_bits(r[j].z * rinv * wv[j].z) | (f32_to_bf16_bits(r[j].w * rinv * wv[j].w) << 16);
+            reinterpret_cast<uint2 *>(y)[i] = make_uint2(lo, hi);
+        }
+    }
 }
 
 // qkv fp32 = [hq*dh | dh | dh].  Rotates q (all heads) and k at position *pos, writes k and v into the caches
@@ -85,55 +137,102 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(const float *__restrict__ 
 }
 
 // Multi-query decode attention, split over the context.  Workgroup b handles positions [b*CS, (b+1)*CS) of the
-// shared K/V for all hq heads: part[b][h] = (max, sum, out[dh]) of its slice.  dh = 256, hq <= 8, CS = 64.
-constexpr int ATT_CS = 64;
+// shared K/V for all hq heads: part[b][h] = (max, sum, out[dh]) of its slice.  dh <= 256, hq <= 8, CS = 32.
+// Every global load of the workgroup (its K rows, its V columns, q) is issued before the first wait: the
+// kernel is one memory round trip plus a few hundred ALU operations per thread.
+constexpr int ATT_CS = 32;
+constexpr int ATT_MAX_NB = 2048;  // slices the combine kernel can hold weights for (context <= 65536)
 __global__ __launch_bounds__(256) void attn_mqa_partial_kernel(const float *__restrict__ q, const uint16_t *__restrict__ kc,
                                                                const uint16_t *__restrict__ vc, const int32_t *__restrict__ pos,
                                                                float *__restrict__ part, int hq, int dh, int max_ctx) {
     const int ctx = min(max(pos[0], 0), max_ctx - 1) + 1;  // positions 0..pos are valid (the current token was just written)
     const int p0 = blockIdx.x * ATT_CS;
     if (p0 >= ctx) return;
-    const int np = (ctx - p0) < ATT_CS ? (ctx - p0) : ATT_CS;
-    __shared__ float s_sc[8][ATT_CS];
+    __shared__ __attribute__((aligned(16))) float s_sc[8][ATT_CS];  // scores, then probabilities
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const float scale = rsqrtf((float)dh);
-    // scores: wave w handles heads w and w+4; lane l handles position p0+l
-    for (int h = wave; h < hq; h += 4) {
-        float s = -INFINITY;
-        if (lane < np) {
-            const uint16_t *kr = kc + (size_t)(p0 + lane) * dh;
-            const float *qh = q + (size_t)h * dh;
-            float acc = 0.f;
-            for (int j = 0; j < dh; j += 8) {
-                const u32x4 kv = *reinterpret_cast<const u32x4 *>(kr + j);
-                const uint32_t kk[4] = {kv.x, kv.y, kv.z, kv.w};
+    const int half = lane >> 5, c = lane & 31, lpr = dh >> 3;  // 16-byte piece c of a K row; two rows per wave load
+
+    // V: thread t owns column t of every row of the slice (rows beyond the context repeat the last valid one;
+    // their probability is 0)
+    const int col = tid < dh ? tid : dh - 1;
+    uint16_t vv[ATT_CS];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    acc += qh[j + 2 * e] * bf16_bits_to_f32(kk[e] & 0xFFFFu);
-                    acc += qh[j + 2 * e + 1] * bf16_bits_to_f32(kk[e] >> 16);
-                }
-            }
-            s = acc * scale;
+    for (int i = 0; i < ATT_CS; ++i) {
+        const int pi = (p0 + i < ctx) ? p0 + i : ctx - 1;
+        vv[i] = vc[(size_t)pi * dh + col];
+    }
+    // K: wave w owns rows 8w..8w+7 of the slice
+    const int cc = c < lpr ? c : 0;
+    u32x4 kv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int pl = wave * 8 + 2 * i + half;
+        const int pi = (p0 + pl < ctx) ? p0 + pl : ctx - 1;
+        kv[i] = *reinterpret_cast<const u32x4 *>(kc + (size_t)pi * dh + cc * 8);
+    }
+    // q: the lane's 8 columns of every head
+    f32x4 qa[8], qb[8];
+#pragma unroll
+    for (int h = 0; h < 8; ++h) {
+        const float *qh = q + (size_t)(h < hq ? h : 0) * dh + cc * 8;
+        qa[h] = *reinterpret_cast<const f32x4 *>(qh);
+        qb[h] = *reinterpret_cast<const f32x4 *>(qh + 4);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    const bool live = c < lpr;
+    const float scale = rsqrtf((float)dh);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int pl = wave * 8 + 2 * i + half;
+        const uint32_t kk[4] = {kv[i].x, kv[i].y, kv[i].z, kv[i].w};
+        float k8[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            k8[2 * e] = live ? bf16_bits_to_f32(kk[e] & 0xFFFFu) : 0.f;
+            k8[2 * e + 1] = live ? bf16_bits_to_f32(kk[e] >> 16) : 0.f;
         }
-        s_sc[h][lane] = s;
+#pragma unroll
+        for (int h = 0; h < 8; ++h) {
+            float acc = qa[h].x * k8[0] + qa[h].y * k8[1] + qa[h].z * k8[2] + qa[h].w * k8[3] + qb[h].x * k8[4] +
+                        qb[h].y * k8[5] + qb[h].z * k8[6] + qb[h].w * k8[7];
+            for (int o = 16; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);  // stays inside the 32-lane half
+            if (c == 0) s_sc[h][pl] = (p0 + pl < ctx && h < hq) ? acc * scale : -INFINITY;
+        }
     }
     __syncthreads();
-    // per head: max, exp, sum over the slice, then out[dh]: thread t handles column t of V (dh = 256 = blockDim)
-    for (int h = 0; h < hq; ++h) {
-        float mx = -INFINITY;
-        for (int i = 0; i < np; ++i) mx = fmaxf(mx, s_sc[h][i]);
-        float sum = 0.f, o = 0.f;
-        for (int i = 0; i < np; ++i) {
-            const float pr = __expf(s_sc[h][i] - mx);
-            sum += pr;
-            if (tid < dh) o += pr * bf16_bits_to_f32(vc[(size_t)(p0 + i) * dh + tid]);
-        }
-        float *dst = part + ((size_t)blockIdx.x * hq + h) * (dh + 2);
-        if (tid == 0) {
+    {
+        // softmax of the slice: thread -> (head tid/32, position tid%32)
+        const int h = tid >> 5, i = tid & 31;
+        const float s = s_sc[h][i];
+        float mx = s;
+        for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        const float pr = (h < hq) ? __expf(s - mx) : 0.f;  // position p0 is always valid, so mx is finite for real heads
+        float sum = pr;
+        for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+        s_sc[h][i] = pr;
+        if (i == 0 && h < hq) {
+            float *dst = part + ((size_t)blockIdx.x * hq + h) * (dh + 2);
             dst[0] = mx;
             dst[1] = sum;
         }
-        if (tid < dh) dst[2 + tid] = o;
+    }
+    __syncthreads();
+    float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < ATT_CS; i += 4) {
+        const float v0 = bf16_bits_to_f32(vv[i]), v1 = bf16_bits_to_f32(vv[i + 1]), v2 = bf16_bits_to_f32(vv[i + 2]),
+                    v3 = bf16_bits_to_f32(vv[i + 3]);
+#pragma unroll
+        for (int h = 0; h < 8; ++h) {
+            const f32x4 p4 = *reinterpret_cast<const f32x4 *>(&s_sc[h][i]);
+            o[h] += p4.x * v0 + p4.y * v1 + p4.z * v2 + p4.w * v3;
+        }
+    }
+    if (tid < dh) {
+#pragma unroll
+        for (int h = 0; h < 8; ++h)
+            if (h < hq) part[((size_t)blockIdx.x * hq + h) * (dh + 2) + 2 + tid] = o[h];
     }
 }
 
@@ -141,16 +240,26 @@ __global__ __launch_bounds__(256) void attn_mqa_partial_kernel(const float *__re
 __global__ __launch_bounds__(256) void attn_mqa_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ pos,
                                                                uint16_t *__restrict__ out, int hq, int dh, int max_ctx) {
     const int ctx = min(max(pos[0], 0), max_ctx - 1) + 1, nb = (ctx + ATT_CS - 1) / ATT_CS, h = blockIdx.x, tid = threadIdx.x;
-    float M = -INFINITY;
-    for (int b = 0; b < nb; ++b) M = fmaxf(M, part[((size_t)b * hq + h) * (dh + 2)]);
-    float den = 0.f, num = 0.f;
-    for (int b = 0; b < nb; ++b) {
-        const float *src = part + ((size_t)b * hq + h) * (dh + 2);
-        const float f = __expf(src[0] - M);
-        den += f * src[1];
-        if (tid < dh) num += f * src[2 + tid];
+    __shared__ float s_f[ATT_MAX_NB];
+    __shared__ float scratch[4];
+    const size_t stride = (size_t)hq * (dh + 2);
+    const float *ph = part + (size_t)h * (dh + 2);
+    float m = -INFINITY;
+    for (int b = tid; b < nb; b += 256) m = fmaxf(m, ph[b * stride]);
+    const float M = block_max(m, scratch);
+    float den = 0.f;
+    for (int b = tid; b < nb; b += 256) {
+        const float f = __expf(ph[b * stride] - M);
+        s_f[b] = f;
+        den += f * ph[b * stride + 1];
     }
-    if (tid < dh) out[(size_t)h * dh + tid] = (uint16_t)f32_to_bf16_bits(num / den);
+    den = block_sum(den, scratch);  // its barriers also publish s_f
+    if (tid < dh) {
+        float num = 0.f;
+#pragma unroll 8
+        for (int b = 0; b < nb; ++b) num += s_f[b] * ph[b * stride + 2 + tid];
+        out[(size_t)h * dh + tid] = (uint16_t)f32_to_bf16_bits(num / den);
+    }
 }
 
 // h = bf16( gelu_tanh(g) * u ), gu = [g(F) | u(F)] fp32
@@ -233,8 +342,27 @@ int embed_launch(const int32_t *token, const uint8_t *wp, const uint16_t *sc, fl
     return hip_check(hipGetLastError(), "embed launch");
 }
 
-int add_rmsnorm_launch(float *res, const float *delta, const float *w, uint16_t *y, int d, float eps, hipStream_t st) {
-    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(256), 0, st, res, delta, w, y, d, eps);
+template <int NV>
+static void add_rmsnorm_vec_launch(float *res, const float *delta, int nd, const float *w, uint16_t *y, int d, float eps,
+                                   hipStream_t st) {
+    switch (nd) {
+        case 0: hipLaunchKernelGGL((add_rmsnorm_vec_kernel<NV, 0>), dim3(1), dim3(256), 0, st, res, delta, w, y, d, eps); break;
+        case 1: hipLaunchKernelGGL((add_rmsnorm_vec_kernel<NV, 1>), dim3(1), dim3(256), 0, st, res, delta, w, y, d, eps); break;
+        case 2: hipLaunchKernelGGL((add_rmsnorm_vec_kernel<NV, 2>), dim3(1), dim3(256), 0, st, res, delta, w, y, d, eps); break;
+        default: hipLaunchKernelGGL((add_rmsnorm_vec_kernel<NV, 4>), dim3(1), dim3(256), 0, st, res, delta, w, y, d, eps); break;
+    }
+}
+
+int add_rmsnorm_launch(float *res, const float *delta, int nd, const float *w, uint16_t *y, int d, float eps, hipStream_t st) {
+    const bool vec = (d % 4 == 0) && d <= 4096 && (nd == 0 || nd == 1 || nd == 2 || nd == 4) &&
+                     ((reinterpret_cast<uintptr_t>(res) | reinterpret_cast<uintptr_t>(delta) | reinterpret_cast<uintptr_t>(w)) & 15u) == 0 &&
+                     (reinterpret_cast<uintptr_t>(y) & 7u) == 0;
+    if (!vec)
+        hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(1), dim3(256), 0, st, res, delta, nd, w, y, d, eps);
+    else if (d <= 2048)
+        add_rmsnorm_vec_launch<2>(res, delta, nd, w, y, d, eps, st);
+    else
+        add_rmsnorm_vec_launch<4>(res, delta, nd, w, y, d, eps, st);
     return hip_check(hipGetLastError(), "add_rmsnorm launch");
 }
 

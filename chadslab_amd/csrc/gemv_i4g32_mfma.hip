@@ -68,7 +68,7 @@ struct GemvCfg {
 template <int MT, int HP, int S, int RBW, int D, int KC>
 __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) void gemv_i4g32_mfma_kernel(
     const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
-    float *__restrict__ y, int N, int K) {
+    float *__restrict__ y, int N, int K, int kspan) {
     typedef GemvCfg<MT, HP, S, RBW, KC> C;
     constexpr int M = MT, MP = C::MP, MPASS = C::MPASS, P = C::P, KS = C::KS, T = C::T, XI = C::XI;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -108,7 +108,11 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
     const int srow_l = lane / C::SC_PPR, spiece = lane % C::SC_PPR;  // lanes beyond P rows repeat the last row
     const int srow = (n0 + srow_l < N) ? n0 + srow_l : N - 1;
 
-    for (int kc0 = 0; kc0 < K; kc0 += KC) {
+    // blockIdx.y selects a K range of kspan (a multiple of KC, or all of K) whose partial sums go to their own
+    // [M,N] block of y: the split-K form for matrices with too few rows to fill the chip
+    const int kbeg = blockIdx.y * kspan, kend = (kbeg + kspan < K) ? kbeg + kspan : K;
+    y += (size_t)blockIdx.y * M * N;
+    for (int kc0 = kbeg; kc0 < kend; kc0 += KC) {
         // 1. activation loads FIRST.  Piece `it` = tid + T*q of pass p: row m = it / 512, i8 = it % 512.
         u32x4 xr[MP][XI];
 #pragma unroll
@@ -240,7 +244,7 @@ int gemv_i4g32_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, flo
 
 template <int MT, int HP, int S, int RBW, int D, int KC = 4096>
 static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K,
-                       hipStream_t st) {
+                       hipStream_t st, int ksplit = 1) {
     typedef GemvCfg<MT, HP, S, RBW, KC> C;
     static bool attr_set = false;
     if (!attr_set) {
@@ -249,8 +253,8 @@ static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc,
         attr_set = true;
     }
     const int units = (N + C::UR - 1) / C::UR;
-    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC>), dim3((units + RBW - 1) / RBW), dim3(256 * RBW), C::TOTAL,
-                       st, x, wp, sc, y, N, K);
+    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC>), dim3((units + RBW - 1) / RBW, ksplit), dim3(256 * RBW),
+                       C::TOTAL, st, x, wp, sc, y, N, K, K / ksplit);
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma launch");
 }
 
@@ -283,6 +287,13 @@ int gemv_i4g32_mfma_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_
         if (rc != 0) return rc;
     }
     return 0;
+}
+
+// Split-K form, M = 1: part s of y_parts [ksplit, N] holds the sum over k in [s*K/ksplit, (s+1)*K/ksplit).
+// K / ksplit must be a multiple of the 4096-wide chunk.
+int gemv_i4g32_splitk_launch(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y_parts, int N, int K,
+                             int ksplit, hipStream_t st) {
+    return launch_mfma<1, 4, 8, 1, 3>(x, wp, sc, y_parts, N, K, st, ksplit);
 }
 
 }  // namespace chadq

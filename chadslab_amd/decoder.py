@@ -69,7 +69,9 @@ class QuantDecoder:
         self.x, self.xn = z(c.d, f32), z(c.d, bf16)
         self.qkv, self.q = z((c.hq + 2) * c.dh, f32), z(c.hq * c.dh, f32)
         self.att, self.ao = z(c.hq * c.dh, bf16), z(c.d, f32)
-        self.gu, self.h, self.dn = z(2 * c.ffn, f32), z(c.ffn, bf16), z(c.d, f32)
+        # the down projection has few rows and a long K: split it over K when that fills the chip better
+        self.ksplit = next((s for s in (4, 2) if c.ffn % (s * 4096) == 0), 1)
+        self.gu, self.h, self.dn = z(2 * c.ffn, f32), z(c.ffn, bf16), z(self.ksplit * c.d, f32)
         self.logits = z(c.vocab, f32)
         self.part = z(self.lib.chadq_attn_decode_mqa_workspace_floats(c.hq, c.dh, c.max_ctx), f32)
         self.scratch = z(512, f32)
@@ -87,7 +89,8 @@ class QuantDecoder:
                                              1, qw.N, qw.K, self._s()), "chadq_gemv_i4g32")
 
     def _norm(self, delta, w):
-        _lib.check(self.lib.chadq_add_rmsnorm_bf16(self.x.data_ptr(), delta.data_ptr() if delta is not None else None,
+        nd = 0 if delta is None else delta.numel() // self.cfg.d
+        _lib.check(self.lib.chadq_add_rmsnorm_bf16(self.x.data_ptr(), delta.data_ptr() if delta is not None else None, nd,
                                                    w.data_ptr(), self.xn.data_ptr(), self.cfg.d, self.cfg.eps, self._s()),
                    "chadq_add_rmsnorm_bf16")
 
@@ -110,7 +113,12 @@ class QuantDecoder:
             self._norm(self.ao, L["ln2"])
             self._gemv(self.xn, L["wgu"], self.gu)
             _lib.check(lib.chadq_geglu_bf16(self.gu.data_ptr(), self.h.data_ptr(), c.ffn, s), "chadq_geglu_bf16")
-            self._gemv(self.h, L["wd"], self.dn)
+            if self.ksplit > 1:
+                _lib.check(lib.chadq_gemv_i4g32_splitk(self.h.data_ptr(), L["wd"].packed.data_ptr(), L["wd"].scale.data_ptr(),
+                                                       self.dn.data_ptr(), c.d, c.ffn, self.ksplit, s),
+                           "chadq_gemv_i4g32_splitk")
+            else:
+                self._gemv(self.h, L["wd"], self.dn)
             pending = self.dn
         self._norm(pending, self.w["lnf"])
         self._gemv(self.xn, self.w["emb"], self.logits)

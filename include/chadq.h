@@ -82,6 +82,14 @@ int chadq_gemv_i4g32(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *
                      int K, void *stream);
 
 /*
+ * Split-K form of the M = 1 product for matrices with few rows and long K (a down projection): y_parts fp32
+ * [ksplit, N], part s = the sum over k in [s*K/ksplit, (s+1)*K/ksplit); the caller adds the parts
+ * (chadq_add_rmsnorm_bf16 does).  K % (ksplit*4096) == 0; x, wp and scale 16-byte aligned.
+ */
+int chadq_gemv_i4g32_splitk(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *scale_f16, float *y_parts, int N,
+                            int K, int ksplit, void *stream);
+
+/*
  * y[m,n] = scale[n] * sum_k x[m,k] * W[n,k]                                 (config 0)
  * x fp32 [M,K], W int8 [N,K], scale fp32 [N], y fp32 [M,N], 1 <= M <= 16, K % 16 == 0.
  */
@@ -139,8 +147,11 @@ int chadq_moe_ffn_i4g32(const uint16_t *x_bf16, const float *logits, const chadq
 int chadq_embed_i4g32(const int32_t *token, const uint8_t *wp, const uint16_t *scale_f16, float *x, int d, int V,
                       void *stream);
 
-/* res[d] += delta[d] (skipped if delta is NULL); y[d] = bf16( res / sqrt(mean(res^2) + eps) * w ). */
-int chadq_add_rmsnorm_bf16(float *res, const float *delta, const float *w, uint16_t *y_bf16, int d, float eps,
+/*
+ * res[d] += delta[0][d] + ... + delta[n_delta-1][d] (delta fp32 [n_delta, d]; nothing is added or written if delta is
+ * NULL or n_delta is 0); y[d] = bf16( res / sqrt(mean(res^2) + eps) * w ).
+ */
+int chadq_add_rmsnorm_bf16(float *res, const float *delta, int n_delta, const float *w, uint16_t *y_bf16, int d, float eps,
                            void *stream);
 
 /*
@@ -156,7 +167,7 @@ size_t chadq_attn_decode_mqa_workspace_floats(int hq, int dh, int max_ctx);
 
 /*
  * Multi-query decode attention over cache rows 0..pos[0]: out bf16 [hq*dh] = softmax(q k^T / sqrt(dh)) v per head,
- * all heads sharing one K/V.  hq <= 8, dh <= 256 and a multiple of 8.
+ * all heads sharing one K/V.  hq <= 8, dh <= 256 and a multiple of 8, max_ctx <= 65536; q and kcache 16-byte aligned.
  */
 int chadq_attn_decode_mqa(const float *q, const uint16_t *kcache_bf16, const uint16_t *vcache_bf16, const int32_t *pos,
                           float *workspace, uint16_t *out_bf16, int hq, int dh, int max_ctx, void *stream);

@@ -54,16 +54,52 @@ def test_add_rmsnorm(lib, d):
     w = (1 + 0.1 * r.standard_normal(d)).astype(np.float32)
     tr, td, tw = dev(res), dev(delta), dev(w)
     y = torch.zeros(d, dtype=torch.bfloat16, device=DEV)
-    chk(lib.chadq_add_rmsnorm_bf16(tr.data_ptr(), td.data_ptr(), tw.data_ptr(), y.data_ptr(), d, 1e-6, stream()), "norm")
+    chk(lib.chadq_add_rmsnorm_bf16(tr.data_ptr(), td.data_ptr(), 1, tw.data_ptr(), y.data_ptr(), d, 1e-6, stream()), "norm")
     want_res = res + delta
     assert np.array_equal(tr.cpu().numpy(), want_res)
     want = O.rmsnorm(want_res, w, 1e-6)
     assert O.rel_l2(O.bf16_to_f32(bits(y)), want) < 5e-3  # bf16 rounding of the output
     # delta = NULL leaves the residual alone
     tr2 = dev(res)
-    chk(lib.chadq_add_rmsnorm_bf16(tr2.data_ptr(), None, tw.data_ptr(), y.data_ptr(), d, 1e-6, stream()), "norm")
+    chk(lib.chadq_add_rmsnorm_bf16(tr2.data_ptr(), None, 0, tw.data_ptr(), y.data_ptr(), d, 1e-6, stream()), "norm")
     assert np.array_equal(tr2.cpu().numpy(), res)
     assert O.rel_l2(O.bf16_to_f32(bits(y)), O.rmsnorm(res, w, 1e-6)) < 5e-3
+
+
+@pytest.mark.parametrize("d,nd", [(2048, 2), (2048, 4), (4096, 4), (3072, 3), (100, 5)])
+def test_add_rmsnorm_sums_partial_vectors_in_order(lib, d, nd):
+    r = rng(d + nd)
+    res = r.standard_normal(d).astype(np.float32)
+    delta = r.standard_normal((nd, d)).astype(np.float32)
+    w = (1 + 0.1 * r.standard_normal(d)).astype(np.float32)
+    tr, td, tw = dev(res), dev(delta), dev(w)
+    y = torch.zeros(d, dtype=torch.bfloat16, device=DEV)
+    chk(lib.chadq_add_rmsnorm_bf16(tr.data_ptr(), td.data_ptr(), nd, tw.data_ptr(), y.data_ptr(), d, 1e-6, stream()), "norm")
+    want = res.copy()
+    for j in range(nd):
+        want = want + delta[j]  # fp32, in order: the residual must match bit for bit
+    assert np.array_equal(tr.cpu().numpy(), want)
+    assert O.rel_l2(O.bf16_to_f32(bits(y)), O.rmsnorm(want, w, 1e-6)) < 5e-3
+
+
+@pytest.mark.parametrize("n,k,ksplit", [(2048, 16384, 4), (2048, 16384, 2), (100, 8192, 2), (33, 4096, 1)])
+def test_gemv_splitk_parts(lib, n, k, ksplit):
+    r = rng(n + k + ksplit)
+    u = r.integers(0, 16, (n, k), dtype=np.uint8)
+    packed = (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8)
+    s = r.lognormal(-5, 0.5, (n, k // 32)).astype(np.float16)
+    xb = O.f32_to_bf16(r.standard_normal((1, k)).astype(np.float32))
+    tp_, ts, tx = dev(packed), dev(s), bf16_tensor(xb.reshape(-1))
+    parts = torch.zeros(ksplit * n, dtype=torch.float32, device=DEV)
+    chk(lib.chadq_gemv_i4g32_splitk(tx.data_ptr(), tp_.data_ptr(), ts.data_ptr(), parts.data_ptr(), n, k, ksplit, stream()),
+        "splitk")
+    got = parts.cpu().numpy().reshape(ksplit, n)
+    kp = k // ksplit
+    for j in range(ksplit):
+        want = O.qgemm_int4g32_f64(xb[:, j * kp:(j + 1) * kp], packed[:, j * kp // 2:(j + 1) * kp // 2], s[:, j * kp // 32:(j + 1) * kp // 32])[0]
+        assert O.rel_l2(got[j], want) < 1e-3
+    with pytest.raises(ValueError):
+        chk(lib.chadq_gemv_i4g32_splitk(tx.data_ptr(), tp_.data_ptr(), ts.data_ptr(), parts.data_ptr(), n, k, 3, stream()), "splitk")
 
 
 @pytest.mark.parametrize("hq,dh,pos", [(8, 256, 0), (8, 256, 2047), (4, 64, 100), (1, 8, 3)])
