@@ -11,7 +11,8 @@ graphs so that Python's per-call cost is not what is measured.
 
 value = algorithmic bytes per launch / average launch duration (HIP events on the launch stream over the
 timed K steps) = the same quantity as roofline.achieved.  Extras: M=4 and M=8, the int8 per-row GEMV
-(config 0) and the prefill dequant-GEMM (config 2, int4 and int8) in TFLOP/s.  cpu_baseline times this build's
+(config 0), the prefill dequant-GEMM (config 2, int4 and int8) in TFLOP/s, the mixture-of-experts FFN (config 3)
+and the Gemma-2B-shaped decode step (config 4) in tokens/s.  cpu_baseline times this build's
 numpy oracle (dequantise to fp32, then sgemv) on the host cores: the reference snapshot has no implementation
 of this path, so there is no reference number to put beside it.
 """
@@ -39,6 +40,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=96)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the side measurements")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run three 256 MiB device copies before the timed region: a kernel of known traffic "
+                         "that hardware-counter runs scale FETCH_SIZE / WRITE_SIZE by")
     return ap.parse_args()
 
 
@@ -95,6 +99,14 @@ def main():
             torch.cuda.synchronize()
             t1 = time.perf_counter()
         return a.elapsed_time(b) * 1000.0 / steps, (t1 - t0) * 1e6 / steps
+
+    if args.calibration_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ------------------------------------------------------------------ config 1 (headline)
     N, K = 14336, 4096
@@ -172,6 +184,72 @@ def main():
             extras[name] = {"us": round(usg, 3), "TFLOPs": round(flop / usg * 1e-6, 1),
                             "frac_bf16_mfma_peak": round(flop / usg * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
+        del x2, y2, q4, q8, p2, s2
+        # config 3: mixture-of-experts FFN, 8 experts, top-2, 256 tokens (weights random bytes: timing only, parity
+        # is the test suite's job)
+        T3, H3, F3, E3 = 256, 4096, 14336, 8
+        g3 = torch.Generator(device=dev)
+        g3.manual_seed(1003)
+
+        def mk(n, k):
+            return QWeightInt4G32(torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev, generator=g3),
+                                  (torch.rand(n, k // 32, device=dev, generator=g3) * 0.01 + 0.002).to(torch.float16))
+
+        experts = [(mk(F3, H3), mk(F3, H3), mk(H3, F3)) for _ in range(E3)]
+        x3 = torch.randn(T3, H3, device=dev, generator=g3).to(torch.bfloat16)
+        z3 = torch.randn(T3, E3, device=dev, generator=g3)
+        with torch.cuda.stream(stream):
+            for _ in range(3):
+                ops.moe_ffn(x3, z3, experts)
+            a3, b3 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a3.record(stream)
+            for _ in range(20):
+                ops.moe_ffn(x3, z3, experts)
+            b3.record(stream)
+            torch.cuda.synchronize()
+        us3 = a3.elapsed_time(b3) * 1000.0 / 20
+        hit = int(torch.unique(ops.moe_route(z3, 2, True)[0]).numel())
+        flop3 = 2.0 * T3 * 2 * 3 * H3 * F3
+        bytes3 = hit * 3 * (F3 * H3 // 2 + F3 * (H3 // 32) * 2)
+        extras["moe_ffn_i4g32_config3"] = {"us": round(us3, 1), "TFLOPs": round(flop3 / us3 * 1e-6, 1),
+                                           "frac_bf16_mfma_peak": round(flop3 / us3 * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                           "experts_hit": hit, "expert_weight_GBps": round(bytes3 / us3 * 1e-3, 1),
+                                           "frac_hbm_peak": round(bytes3 / us3 * 1e-3 / HBM_PEAK_GBS, 4)}
+        del experts, x3, z3
+        torch.cuda.empty_cache()
+        # config 4: decode step, 18 layers, d 2048, 8 query heads x 256, 1 KV head, FFN 16384, vocab 256000, batch 1,
+        # KV cache pre-filled to 2048 positions; 64 graph-replayed greedy steps (context 2048..2111)
+        from chadslab_amd.decoder import DecoderConfig, QuantDecoder, random_weights
+
+        cfg4 = DecoderConfig(max_ctx=4096)
+        w4 = random_weights(cfg4, 1004, dev)
+        with torch.cuda.stream(stream):
+            dec = QuantDecoder(cfg4, w4, dev)
+            for li in range(cfg4.n_layers):
+                dec.kcache[li].normal_()
+                dec.vcache[li].normal_()
+            dec.token.fill_(5)
+            dec.pos.fill_(2040)
+            dec.capture()
+            for _ in range(8):
+                dec.graph.replay()
+            a4, b4 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a4.record(stream)
+            for _ in range(64):
+                dec.graph.replay()
+            b4.record(stream)
+            torch.cuda.synchronize()
+        us4 = a4.elapsed_time(b4) * 1000.0 / 64
+        wbytes = sum(q.packed.numel() + 2 * q.scale.numel() for L in w4["layers"] for q in (L["wqkv"], L["wo"], L["wgu"], L["wd"]))
+        wbytes += w4["emb"].packed.numel() + 2 * w4["emb"].scale.numel()
+        kvbytes = cfg4.n_layers * 2 * 2080 * cfg4.dh * 2
+        extras["decode_step_config4"] = {"us_per_token": round(us4, 1), "tokens_per_s": round(1e6 / us4, 1),
+                                         "bytes_per_token": wbytes + kvbytes, "GBps": round((wbytes + kvbytes) / us4 * 1e-3, 1),
+                                         "frac_hbm_peak": round((wbytes + kvbytes) / us4 * 1e-3 / HBM_PEAK_GBS, 4),
+                                         "context": "2048..2111", "launch": "one HIP graph per token"}
+        del dec, w4
+        torch.cuda.empty_cache()
+
     # ------------------------------------------------------------------ CPU baseline (rank 0, N=1)
     cpu = None
     if not args.no_cpu:
@@ -227,7 +305,7 @@ def main():
                    "algorithmic_bytes_per_launch": gemv_bytes(1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "gemv_i4g32_mfma_kernel<1,1>", "wall_clock_us_per_step": round(wall1, 3)},
+                     "kernel": "gemv_i4g32_mfma_kernel<1,4,8,1,3,4096>", "wall_clock_us_per_step": round(wall1, 3)},
         "cpu_baseline": cpu,
         "parity": parity,
         "extras": extras,
