@@ -29,6 +29,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16
+# HBM bytes per launch of the headline kernel from hardware counters (FETCH_SIZE, WRITE_SIZE, each scaled by what a
+# 256 MiB copy reads for it); the counter runs are summarised in profiles/gemv_i4g32_m1_config1_hbm_traffic.txt
+GEMV_M1_TRAFFIC_BYTES = 33234000
 N_COPIES = 12
 SEG = 48                     # launches per captured graph
 
@@ -304,7 +307,7 @@ def main():
                    "M": 1, "N": N, "K": K, "weight_copies_rotated": N_COPIES, "launch": "HIP graph replay, %d launches per graph" % SEG,
                    "algorithmic_bytes_per_launch": gemv_bytes(1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_M1_TRAFFIC_BYTES,
                      "kernel": "gemv_i4g32_mfma_kernel<1,4,8,1,3,4096>", "wall_clock_us_per_step": round(wall1, 3)},
         "cpu_baseline": cpu,
         "parity": parity,
