@@ -72,6 +72,23 @@ __device__ __forceinline__ bf16x2 as_bf16x2(uint32_t v) {
     return r;
 }
 
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+
+__device__ __forceinline__ f16x2 as_f16x2(uint32_t v) {
+    f16x2 r;
+    __builtin_memcpy(&r, &v, 4);
+    return r;
+}
+
+__device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
+    f32x2 f = {a, b};
+    bf16x2 h = __builtin_convertvector(f, bf16x2);
+    uint32_t r;
+    __builtin_memcpy(&r, &h, 4);
+    return r;
+}
+
 // One 32-bit word of packed weights = 8 nibbles u0..u7 (u0 lowest).  Returns four registers of bf16
 // pairs holding 128+u: p[i] = (128+u_i , 128+u_{i+4}), i = 0..3.  Exact: 128+u <= 143 fits bf16.
 __device__ __forceinline__ void unpack8_magic(uint32_t w, uint32_t p[4]) {

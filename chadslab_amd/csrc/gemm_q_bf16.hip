@@ -24,23 +24,6 @@
 
 namespace chadq {
 
-typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
-typedef __attribute__((ext_vector_type(2))) float f32x2;
-
-__device__ __forceinline__ f16x2 as_f16x2(uint32_t v) {
-    f16x2 r;
-    __builtin_memcpy(&r, &v, 4);
-    return r;
-}
-
-__device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
-    f32x2 f = {a, b};
-    bf16x2 h = __builtin_convertvector(f, bf16x2);
-    uint32_t r;
-    __builtin_memcpy(&r, &h, 4);
-    return r;
-}
-
 struct FmtI4G32 {
     static constexpr int KL = 32;  // k per 16-byte weight load
     typedef uint16_t scale_t;

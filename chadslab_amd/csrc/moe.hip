@@ -5,8 +5,9 @@
 // Everything runs on the caller's stream without a host round trip: the router kernel also sorts the
 // (token, slot) pairs by expert (stable: by pair index inside an expert) and writes the per-expert descriptors
 // of three grouped GEMM launches (gate, up: fp32 out; down: fp32 out), whose row counts therefore never
-// leave the GPU.  Gate/up/down are the dequant-GEMM kernel in grouped mode; the small kernels here are the
-// gather, the SiLU gate and the weighted combine.
+// leave the GPU.  Gate/up/down run on the skinny grouped kernel (gate and up fused with the SiLU gate, down split
+// over K) when H and F are multiples of 256, else on the prefill dequant-GEMM kernel in grouped mode with a
+// separate SiLU kernel; the small kernels here are the gather, the SiLU gate and the weighted combine.
 #include "chadq_common.h"
 
 namespace chadq {
@@ -28,10 +29,15 @@ struct MoeWs {  // workspace carved up on the host
     uint16_t *xs;        // [P,H] gathered activations (bf16)
     float *g, *u;        // [P,F]
     uint16_t *h;         // [P,F] bf16
-    float *yp;           // [P,H]
+    float *yp;           // [MOE_KSPLIT][P,H] partial down projections
 };
 
+constexpr int MOE_KSPLIT = 2;
+
 int gemm_i4g32_grouped(const GemmGroup *groups, int ngroups, int m_max, int N, int K, bool out_f32, hipStream_t st);
+bool gemm_skinny_ok(int H, int F);
+int gemm_skinny_gateup(const GemmGroup *groups, int E, int m_max, int F, int H, hipStream_t st);
+int gemm_skinny_down(const GemmGroup *groups, int E, int m_max, int H, int F, int ksplit, size_t ysplit_stride, hipStream_t st);
 
 // One workgroup.  Phase 1: softmax + top-k per token.  Phase 2: stable counting sort of the pairs by expert.
 // Phase 3: descriptors.  idx/w may be the caller's arrays (chadq_moe_route) with everything else null.
@@ -145,17 +151,19 @@ __global__ __launch_bounds__(256) void moe_act_kernel(const float *__restrict__ 
     }
 }
 
-// y[t] = bf16( sum_j w[t,j] * yp[pos[t*top_k+j]] ), slots in order; 4 columns per thread
+// y[t] = bf16( sum_j w[t,j] * sum_s yp[s][pos[t*top_k+j]] ), slots in order, K-split parts in order; 4 columns per thread
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restrict__ yp, const int32_t *__restrict__ pos,
                                                           const float *__restrict__ w, uint16_t *__restrict__ y, int T,
-                                                          int H, int top_k) {
+                                                          int H, int top_k, int nsplit, size_t split_stride) {
     const int q = H / 4;
     const int64_t total = (int64_t)T * q, stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
         const int t = (int)(i / q), c = (int)(i % q);
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         for (int j = 0; j < top_k; ++j) {
-            const f32x4 v = reinterpret_cast<const f32x4 *>(yp + (size_t)pos[t * top_k + j] * H)[c];
+            f32x4 v = reinterpret_cast<const f32x4 *>(yp + (size_t)pos[t * top_k + j] * H)[c];
+            for (int sp = 1; sp < nsplit; ++sp)
+                v += reinterpret_cast<const f32x4 *>(yp + sp * split_stride + (size_t)pos[t * top_k + j] * H)[c];
             acc += v * w[t * top_k + j];
         }
         u32x2 o = {f32_to_bf16_bits(acc.x) | (f32_to_bf16_bits(acc.y) << 16), f32_to_bf16_bits(acc.z) | (f32_to_bf16_bits(acc.w) << 16)};
@@ -185,7 +193,7 @@ static size_t moe_layout(uint8_t *base, int T, int H, int F, int E, int top_k, M
     w.g = (float *)take(P * F * 4);
     w.u = (float *)take(P * F * 4);
     w.h = (uint16_t *)take(P * F * 2);
-    w.yp = (float *)take(P * H * 4);
+    w.yp = (float *)take(P * H * 4 * MOE_KSPLIT);
     if (ws) *ws = w;
     return o;
 }
@@ -218,12 +226,26 @@ int moe_ffn_i4g32_launch(const uint16_t *x, const float *logits, const chadq_moe
     hipLaunchKernelGGL(moe_gather_kernel, dim3(512), dim3(256), 0, st, x, ws.tok, ws.xs, P, H);
     int rc = hip_check(hipGetLastError(), "moe route/gather launch");
     if (rc) return rc;
-    rc = gemm_i4g32_grouped(ws.groups, 2 * E, m_max, F, H, true, st);  // gate and up: fp32 [P,F] each
-    if (rc) return rc;
-    hipLaunchKernelGGL(moe_act_kernel, dim3(2048), dim3(256), 0, st, ws.g, ws.u, ws.h, (int64_t)P * F / 4);
-    rc = gemm_i4g32_grouped(ws.groups + 2 * E, E, m_max, H, F, true, st);  // down: fp32 [P,H]
-    if (rc) return rc;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(1024), dim3(256), 0, st, ws.yp, ws.pos, ws.w, y, T, H, top_k);
+    int nsplit = 1;
+    bool aligned = true;  // the skinny kernel loads scales 16 bytes at a time
+    for (int e = 0; e < E; ++e)
+        aligned = aligned && aligned16(experts[e].wg) && aligned16(experts[e].sg) && aligned16(experts[e].wu) &&
+                  aligned16(experts[e].su) && aligned16(experts[e].wd) && aligned16(experts[e].sd);
+    if (aligned && gemm_skinny_ok(H, F)) {
+        rc = gemm_skinny_gateup(ws.groups, E, m_max, F, H, st);  // h = bf16(silu(gate) * up), [P,F]
+        if (rc) return rc;
+        nsplit = (F % (256 * MOE_KSPLIT) == 0) ? MOE_KSPLIT : 1;
+        rc = gemm_skinny_down(ws.groups, E, m_max, H, F, nsplit, (size_t)P * H, st);  // fp32 parts [nsplit][P,H]
+        if (rc) return rc;
+    } else {
+        rc = gemm_i4g32_grouped(ws.groups, 2 * E, m_max, F, H, true, st);  // gate and up: fp32 [P,F] each
+        if (rc) return rc;
+        hipLaunchKernelGGL(moe_act_kernel, dim3(2048), dim3(256), 0, st, ws.g, ws.u, ws.h, (int64_t)P * F / 4);
+        rc = gemm_i4g32_grouped(ws.groups + 2 * E, E, m_max, H, F, true, st);  // down: fp32 [P,H]
+        if (rc) return rc;
+    }
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(1024), dim3(256), 0, st, ws.yp, ws.pos, ws.w, y, T, H, top_k, nsplit,
+                       (size_t)P * H);
     return hip_check(hipGetLastError(), "moe act/combine launch");
 }
 

@@ -306,7 +306,8 @@ def test_moe_golden(ops):
     assert O.rel_l2(O.bf16_to_f32(bits(y)), O.bf16_to_f32(g["y_bf16"])) <= TOL_BF16
 
 
-@pytest.mark.parametrize("t,h,f,e,top_k", [(256, 512, 1024, 8, 2), (37, 128, 160, 3, 1), (64, 256, 256, 1, 1), (130, 256, 512, 16, 4)])
+@pytest.mark.parametrize("t,h,f,e,top_k", [(256, 512, 1024, 8, 2), (37, 128, 160, 3, 1), (64, 256, 256, 1, 1), (130, 256, 512, 16, 4),
+                                           (300, 256, 512, 2, 2), (33, 256, 768, 8, 2), (200, 512, 512, 3, 1)])
 def test_moe_ffn(ops, t, h, f, e, top_k):
     host, dev = _experts(80 + t, e, h, f)
     r = rng(81 + t)
