@@ -89,6 +89,25 @@ __device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
     return r;
 }
 
+// s_waitcnt with only the vector-memory counter set (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);
+}
+
+// 16 (or 2) bytes per lane from global memory straight into LDS at `lds_dst` + lane * 16 (lane * 4 for 2 bytes);
+// lds_dst must be the same for the whole wave.  Completion is tracked by vmcnt; the compiler inserts no wait
+// for later LDS reads of that data, so callers wait explicitly.
+__device__ __forceinline__ void dma16_to_lds(const void *gsrc, void *lds_dst) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gsrc,
+                                     (__attribute__((address_space(3))) void *)lds_dst, 16, 0, 0);
+}
+__device__ __forceinline__ void dma2_to_lds(const void *gsrc, void *lds_dst) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gsrc,
+                                     (__attribute__((address_space(3))) void *)lds_dst, 2, 0, 0);
+}
+
 // One 32-bit word of packed weights = 8 nibbles u0..u7 (u0 lowest).  Returns four registers of bf16
 // pairs holding 128+u: p[i] = (128+u_i , 128+u_{i+4}), i = 0..3.  Exact: 128+u <= 143 fits bf16.
 __device__ __forceinline__ void unpack8_magic(uint32_t w, uint32_t p[4]) {

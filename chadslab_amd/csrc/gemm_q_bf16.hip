@@ -98,13 +98,6 @@ struct Tile {
 template <typename TL>
 __device__ __forceinline__ int swz(int row, int piece) { return piece ^ ((row / TL::RPL) % TL::PPR); }
 
-// s_waitcnt with only the vector-memory counter set (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);
-}
-
 // GUARD = false assumes K is a multiple of the workgroup's k step (no range checks in the loop).
 // OUTF32: y is fp32 [M,N] instead of bf16.  groups != nullptr: grouped launch, blockIdx.y selects a descriptor
 // (activations, weights, output and row count of one group; N and K are common) - this is how the MoE expert

@@ -1,8 +1,8 @@
 // Grouped "skinny" dequant-GEMM for the mixture-of-experts FFN: few activation rows (the tokens routed to one
 // expert, tens to a hundred or so) against many int4 group-32 weight rows.  The prefill tile (128 x 64) is the
 // wrong shape here: half of its rows are padding and every 64 weight rows re-read the whole activation panel.
-// This kernel turns the tile around: one workgroup takes up to 128 tokens of one expert and 256 weight rows,
-//   - the activation tile (32*MB rows x 64 k per iteration, MB = 1..4 from the expert's actual row count) goes
+// This kernel turns the tile around: one workgroup takes up to 96 tokens of one expert and 256 weight rows,
+//   - the activation tile (32*MB rows x 64 k per iteration, MB = 1..3 from the expert's actual row count) goes
 //     through LDS once per workgroup and is shared by the four waves (XOR-swizzled 16-byte pieces);
 //   - each wave owns 64 weight rows: its lanes stream them straight from global memory (16 B = one group of 32
 //     nibbles per load), dequantise in registers (fp16 magic number, one FMA per element, RNE to bf16) and feed
@@ -18,7 +18,7 @@
 
 namespace chadq {
 
-constexpr int SK_MT = 128;  // tokens per workgroup tile
+constexpr int SK_MT = 96;   // tokens per workgroup tile
 constexpr int SK_KI = 64;   // k per iteration
 
 struct SkDequant {
@@ -42,6 +42,24 @@ struct SkDequant {
     }
 };
 
+// Operand supply: everything comes global -> LDS by DMA, ahead of its use, so that memory latency is covered by
+// bytes in flight rather than by registers or occupancy:
+//   activation ring (shared by the workgroup): 3 stages of 32*SK_MB rows x 64 k, each wave fetches a quarter,
+//     two iterations ahead;
+//   weight ring (private to a wave): 2 slots of 128 k: 64 rows x 64 B of packed weights fetched as 4 DMA
+//     instructions of 16 rows x 64 contiguous bytes (whole 64-byte sectors: fetching 32 B per row per iteration
+//     made HBM traffic 2.5 x the weight bytes), plus 64 rows x 16 B of group scales; a slot serves two
+//     iterations and is refilled right after its last use, one slot (two iterations) ahead.
+// Every wave issues MB DMA instructions per iteration plus 5 on even ones; memory returns in order, so the waits
+// below count how many younger requests may still be outstanding.  Past the end of K the requests repeat the
+// first addresses so the counts stay uniform (their slots are never read).
+constexpr int SK_MB = SK_MT / 32;
+constexpr int SK_ASTAGE = SK_MB * 32 * 128;
+constexpr int SK_A_BYTES = 3 * SK_ASTAGE;
+constexpr int SK_BSLOT = 64 * 64 + 64 * 16;
+constexpr int SK_B_WAVE = 2 * SK_BSLOT;
+constexpr int SK_LDS = SK_A_BYTES + 4 * SK_B_WAVE;
+
 template <int MODE, int MB>
 __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, const uint8_t *__restrict__ w0,
                                             const uint16_t *__restrict__ s0, const uint8_t *__restrict__ w1,
@@ -50,36 +68,45 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nl = lane & 31, kq = lane >> 5;
-    constexpr int STAGE = MB * 32 * 128;  // bytes of one activation stage
 
-    // weight rows of this lane
-    const uint8_t *wrow[2];
-    const uint16_t *srow[2];
-    if (MODE == 1) {
-        const int f = n0 + wave * 32 + nl;
-        wrow[0] = w0 + (size_t)f * (K >> 1);
-        wrow[1] = w1 + (size_t)f * (K >> 1);
-        srow[0] = s0 + (size_t)f * (K >> 5);
-        srow[1] = s1 + (size_t)f * (K >> 5);
-    } else {
+    // wave-local weight row rho (0..63) -> matrix row: MODE 0: n0 + 64*wave + rho; MODE 1: rows 0..31 are gate
+    // features n0 + 32*wave + rho, rows 32..63 the same features of the up matrix
+    auto wptr = [&](int rho) -> const uint8_t * {
+        if (MODE == 1) return (rho < 32 ? w0 : w1) + (size_t)(n0 + wave * 32 + (rho & 31)) * (K >> 1);
+        return w0 + (size_t)(n0 + wave * 64 + rho) * (K >> 1);
+    };
+    auto sptr = [&](int rho) -> const uint16_t * {
+        if (MODE == 1) return (rho < 32 ? s0 : s1) + (size_t)(n0 + wave * 32 + (rho & 31)) * (K >> 5);
+        return s0 + (size_t)(n0 + wave * 64 + rho) * (K >> 5);
+    };
+    // weight fetch: DMA instruction i, lane l -> row 16i + l/4, LDS position l%4, which holds 16-byte piece
+    // (l%4) ^ ((row >> 1) & 3) of the row's 64 bytes (bank-conflict-free read-back)
+    const uint8_t *wsrc[4];
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-            const int n = n0 + wave * 64 + nb * 32 + nl;
-            wrow[nb] = w0 + (size_t)n * (K >> 1);
-            srow[nb] = s0 + (size_t)n * (K >> 5);
-        }
+    for (int i = 0; i < 4; ++i) {
+        const int rho = 16 * i + (lane >> 2);
+        wsrc[i] = wptr(rho) + (((lane & 3) ^ ((rho >> 1) & 3)) << 4);
     }
-    // activation pieces of this thread: piece p of rows r, r+32, ...; rows past the tile repeat its last row
-    const int p = tid & 7, r = tid >> 3;
-    const uint16_t *arow[MB];
-    uint32_t awr[MB];
+    const uint16_t *ssrc = sptr(lane);  // scale fetch: lane l -> row l, 8 groups (256 k)
+    // read-back: lane (nl, kq), block nb -> row nb*32 + nl; half h of the slot -> piece 2h + kq
+    uint32_t brd[2][2];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int rho = nb * 32 + nl;
+            brd[nb][h] = (uint32_t)(rho * 64 + (((2 * h + kq) ^ ((rho >> 1) & 3)) << 4));
+        }
+    // activation pieces this lane requests: DMA instruction i of wave w fills LDS bytes (4i + w) * 1024 + 16 * lane
+    // of a stage, i.e. row rr = (4i + w) * 8 + lane / 8, slot lane % 8, which holds piece slot ^ (rr & 7).  Rows
+    // past the tile repeat its last row (their results are never stored).
+    const uint16_t *asrc[MB];
 #pragma unroll
     for (int i = 0; i < MB; ++i) {
-        const int rr = i * 32 + r, rc = rr < rows ? rr : rows - 1;
-        arow[i] = x + (size_t)(m0 + rc) * K + p * 8;
-        awr[i] = (uint32_t)(rr * 128 + ((p ^ (r & 7)) << 4));
+        const int rr = (4 * i + wave) * 8 + (lane >> 3), rc = rr < rows ? rr : rows - 1;
+        asrc[i] = x + (size_t)(m0 + rc) * K + (((lane & 7) ^ (rr & 7)) << 3);
     }
-    // fragment read offsets: row mb*32+nl, piece kq*4+j lives in slot (kq*4+j) ^ (nl & 7)
+    // fragment read offsets: row mb*32 + nl, piece kq*4 + j lives in slot (kq*4 + j) ^ (nl & 7)
     uint32_t ard[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) ard[j] = (uint32_t)(nl * 128 + (((kq * 4 + j) ^ (nl & 7)) << 4));
@@ -93,90 +120,103 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
             for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
     const uint32_t c_mlo = vgpr_const(0x000F000Fu), c_mhi = vgpr_const(0x00F000F0u), c_magic = vgpr_const(0x64006400u);
-    u32x4 ra[2][MB];          // activation pieces in flight: ra[it & 1] = iteration it
-    u32x4 rb[3][2];           // packed weights: rb[0] = this iteration, rb[1], rb[2] = the next two
-    u32x4 rs_cur[2], rs_nxt[2];  // 8 group scales (256 k) per weight row block
+    uint8_t *bring = lds + SK_A_BYTES + wave * SK_B_WAVE;
+    const int nit = (kend - kbeg) / SK_KI;  // even
 
-    auto load_a = [&](int par, int k0) {
+    auto issue_a = [&](int itn, int stage) {
+        const int k = (itn < nit) ? kbeg + itn * SK_KI : kbeg;
+        uint8_t *adst = lds + stage * SK_ASTAGE + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < MB; ++i) ra[par][i] = *reinterpret_cast<const u32x4 *>(arow[i] + k0);
+        for (int i = 0; i < MB; ++i) dma16_to_lds(asrc[i] + k, adst + i * 4096);
     };
-    auto load_b = [&](int slot, int k0) {
+    auto issue_b = [&](int m, int slot) {  // weights and scales of iterations 2m, 2m+1
+        const int k = (2 * m < nit) ? kbeg + m * 2 * SK_KI : kbeg;
+        uint8_t *bdst = bring + slot * SK_BSLOT;
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) rb[slot][nb] = load_nt_b128(wrow[nb] + ((k0 + 32 * kq) >> 1));
-    };
-    auto load_s = [&](u32x4(&dst)[2], int k0) {
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) dst[nb] = *reinterpret_cast<const u32x4 *>(srow[nb] + (k0 >> 5));
-    };
-    auto store_a = [&](int par, int stage) {
-#pragma unroll
-        for (int i = 0; i < MB; ++i) *reinterpret_cast<u32x4 *>(lds + stage * STAGE + awr[i]) = ra[par][i];
+        for (int i = 0; i < 4; ++i) dma16_to_lds(wsrc[i] + (k >> 1), bdst + i * 1024);
+        dma16_to_lds(ssrc + ((k & ~255) >> 5), bdst + 4096);
     };
 
-    const int nit = (kend - kbeg) / SK_KI;  // a multiple of 4
-    load_s(rs_cur, kbeg);
-    load_a(0, kbeg);
-    load_b(0, kbeg);
-    load_a(1, kbeg + SK_KI);
-    load_b(1, kbeg + SK_KI);
-    store_a(0, 0);
-    __syncthreads();
-
-    for (int it0 = 0; it0 < nit; it0 += 4) {
+    // one iteration (64 k): weights of half `h` of weight slot `bslot`, activations of stage `stage`
+    auto compute = [&](int stage, int bslot, int h, int k) {
+        const uint8_t *bs = bring + bslot * SK_BSLOT;
+        const uint8_t *ab = lds + stage * SK_ASTAGE;
+        const int gi = ((k & 255) >> 5) + kq;  // the lane's group among the 8 whose scales the slot holds
+        u32x4 q[2];
+        uint32_t sbits[2];
+        bf16x8 af[2][MB];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int it = it0 + u, k0 = kbeg + it * SK_KI;
-            const int s = u & 1;
-            // prefetch two iterations ahead; past the end the loads repeat the first iteration (never used)
-            const int k2 = (it + 2 < nit) ? k0 + 2 * SK_KI : kbeg;
-            load_a(s, k2);  // ra[s] (iteration it) went to LDS one iteration ago
-            load_b(2, k2);
-            if (u == 0) load_s(rs_nxt, (it0 + 4 < nit) ? k0 + 4 * SK_KI : kbeg);
-
-            // this iteration's group scale: group 2*u + kq of the 8 held
-            float cs[2][4];
+        for (int nb = 0; nb < 2; ++nb) {
+            q[nb] = *reinterpret_cast<const u32x4 *>(bs + brd[nb][h]);
+            sbits[nb] = *reinterpret_cast<const uint16_t *>(bs + 4096 + (nb * 32 + nl) * 16 + gi * 2);
+        }
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
-                const uint32_t wsel = u == 0 ? rs_cur[nb].x : u == 1 ? rs_cur[nb].y : u == 2 ? rs_cur[nb].z : rs_cur[nb].w;
-                const float sc = f16_bits_to_f32((wsel >> (16 * kq)) & 0xFFFFu);
-                cs[nb][0] = sc;
-                cs[nb][1] = sc * 0.0625f;
-                cs[nb][2] = -1032.f * sc;
-                cs[nb][3] = -72.f * sc;
+        for (int mb = 0; mb < MB; ++mb) af[0][mb] = *reinterpret_cast<const bf16x8 *>(ab + mb * 4096 + ard[0]);
+        __builtin_amdgcn_sched_barrier(0);
+        float cs[2][4];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            const float sc = f16_bits_to_f32(sbits[nb]);
+            cs[nb][0] = sc;
+            cs[nb][1] = sc * 0.0625f;
+            cs[nb][2] = -1032.f * sc;
+            cs[nb][3] = -72.f * sc;
+        }
+        // LDS reads of a step are issued one step ahead of their use, and the dequantisation of step j+1 follows
+        // the MFMAs of step j in program order, so that it runs on the VALU while the matrix core works.
+        bf16x8 bf[2][2];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+            bf[0][nb] = SkDequant::run(q[nb].x, cs[nb][0], cs[nb][1], cs[nb][2], cs[nb][3], c_mlo, c_mhi, c_magic);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (j < 3) {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                    af[(j + 1) & 1][mb] = *reinterpret_cast<const bf16x8 *>(ab + mb * 4096 + ard[j + 1]);
             }
-            const uint8_t *ab = lds + s * STAGE;
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                bf16x8 bf[2];
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb)
+                    acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[j & 1][mb], bf[j & 1][nb], acc[mb][nb], 0, 0, 0);
+            if (j < 3) {
 #pragma unroll
                 for (int nb = 0; nb < 2; ++nb) {
-                    const u32x4 q = rb[0][nb];
-                    const uint32_t wsel = j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
-                    bf[nb] = SkDequant::run(wsel, cs[nb][0], cs[nb][1], cs[nb][2], cs[nb][3], c_mlo, c_mhi, c_magic);
-                }
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) {
-                    const bf16x8 af = *reinterpret_cast<const bf16x8 *>(ab + mb * 4096 + ard[j]);
-#pragma unroll
-                    for (int nb = 0; nb < 2; ++nb)
-                        acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bf[nb], acc[mb][nb], 0, 0, 0);
+                    const uint32_t wsel = j == 0 ? q[nb].y : j == 1 ? q[nb].z : q[nb].w;
+                    bf[(j + 1) & 1][nb] = SkDequant::run(wsel, cs[nb][0], cs[nb][1], cs[nb][2], cs[nb][3], c_mlo, c_mhi, c_magic);
                 }
             }
-            // the next iteration's activations go to the other stage (last read one iteration ago, barrier since)
-            store_a(s ^ 1, s ^ 1);
-            __syncthreads();
-#pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
-                rb[0][nb] = rb[1][nb];
-                rb[1][nb] = rb[2][nb];
-            }
-            if (u == 3) {
-                rs_cur[0] = rs_nxt[0];
-                rs_cur[1] = rs_nxt[1];
-            }
+            __builtin_amdgcn_sched_barrier(0);
         }
+    };
+
+    // request order: A(0) B(0) A(1) | it=0: A(2) B(1) | it=1: A(3) | it=2: A(4) B(2) | ...
+    issue_a(0, 0);
+    issue_b(0, 0);
+    issue_a(1, 1);
+    int st = 0;  // it % 3
+    for (int it = 0; it < nit; it += 2) {
+        const int m = it >> 1, st1 = st == 2 ? 0 : st + 1, st2 = st1 == 2 ? 0 : st1 + 1;
+        // even iteration: needs A(it) and B(m); only A(it+1) is younger
+        wait_vmcnt<MB>();
+        // the bare barrier instruction: __syncthreads() would add a fence that waits for every outstanding
+        // request (vmcnt 0) and with it the whole prefetch
+        __builtin_amdgcn_s_barrier();  // everybody's part of A(it) has landed; everybody is done reading A(it-1)
+        __builtin_amdgcn_sched_barrier(0);
+        issue_a(it + 2, st2);          // into the stage of A(it-1)
+        issue_b(m + 1, (m + 1) & 1);   // into the slot of B(m-1), which this wave finished in iteration it-1
+        compute(st, m & 1, 0, kbeg + it * SK_KI);
+        // odd iteration: needs A(it+1); A(it+2) and B(m+1) are younger
+        wait_vmcnt<MB + 5>();
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        issue_a(it + 3, st);           // into the stage of A(it)
+        compute(st1, m & 1, 1, kbeg + (it + 1) * SK_KI);
+        st = st2;
     }
+    wait_vmcnt<0>();  // the surplus requests of the last iterations must not outlive the workgroup's LDS
 
     // epilogue: lane (nl, kq) holds column nl of rows 8*(v/4) + 4*kq + v%4 of each 32 x 32 block
 #pragma unroll
@@ -227,29 +267,34 @@ __global__ __launch_bounds__(256, 2) void gemm_skinny_i4g32_kernel(const GemmGro
     switch ((rows + 31) >> 5) {
         case 1: skinny_body<MODE, 1>(ga.x, w0, s0, w1, s1, y, m0, rows, n0, N, K, kbeg, kend, lds); break;
         case 2: skinny_body<MODE, 2>(ga.x, w0, s0, w1, s1, y, m0, rows, n0, N, K, kbeg, kend, lds); break;
-        case 3: skinny_body<MODE, 3>(ga.x, w0, s0, w1, s1, y, m0, rows, n0, N, K, kbeg, kend, lds); break;
-        default: skinny_body<MODE, 4>(ga.x, w0, s0, w1, s1, y, m0, rows, n0, N, K, kbeg, kend, lds); break;
+        default: skinny_body<MODE, 3>(ga.x, w0, s0, w1, s1, y, m0, rows, n0, N, K, kbeg, kend, lds); break;
     }
 }
 
-constexpr int SK_LDS = 2 * 4 * 32 * 128;  // two stages of up to 128 rows x 64 k bf16
-
 bool gemm_skinny_ok(int H, int F) { return H % 256 == 0 && F % 256 == 0; }
+
+template <int MODE>
+static int skinny_launch(const GemmGroup *groups, int E, int mtiles, int ntiles, int N, int K, int ksplit, size_t ystride,
+                         hipStream_t st) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_skinny_i4g32_kernel<MODE>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((gemm_skinny_i4g32_kernel<MODE>), dim3(ntiles, E * mtiles, ksplit), dim3(256), SK_LDS, st,
+                       groups, E, N, K, K / ksplit, mtiles, ystride);
+    return hip_check(hipGetLastError(), "gemm_skinny launch");
+}
 
 // gate/up with the SiLU epilogue: h[P,F] bf16 (through the down descriptors' x pointers)
 int gemm_skinny_gateup(const GemmGroup *groups, int E, int m_max, int F, int H, hipStream_t st) {
-    const int mtiles = (m_max + SK_MT - 1) / SK_MT;
-    hipLaunchKernelGGL((gemm_skinny_i4g32_kernel<1>), dim3(F / 128, E * mtiles, 1), dim3(256), SK_LDS, st, groups, E, F, H, H,
-                       mtiles, (size_t)0);
-    return hip_check(hipGetLastError(), "gemm_skinny gate/up launch");
+    return skinny_launch<1>(groups, E, (m_max + SK_MT - 1) / SK_MT, F / 128, F, H, 1, 0, st);
 }
 
 // down: fp32 parts [ksplit][P,H]
 int gemm_skinny_down(const GemmGroup *groups, int E, int m_max, int H, int F, int ksplit, size_t ysplit_stride, hipStream_t st) {
-    const int mtiles = (m_max + SK_MT - 1) / SK_MT;
-    hipLaunchKernelGGL((gemm_skinny_i4g32_kernel<0>), dim3(H / 256, E * mtiles, ksplit), dim3(256), SK_LDS, st, groups, E, H, F,
-                       F / ksplit, mtiles, ysplit_stride);
-    return hip_check(hipGetLastError(), "gemm_skinny down launch");
+    return skinny_launch<0>(groups, E, (m_max + SK_MT - 1) / SK_MT, H / 256, H, F, ksplit, ysplit_stride, st);
 }
 
 }  // namespace chadq
