@@ -32,7 +32,7 @@ struct MoeWs {  // workspace carved up on the host
     float *yp;           // [MOE_KSPLIT][P,H] partial down projections
 };
 
-constexpr int MOE_KSPLIT = 2;
+constexpr int MOE_KSPLIT = 4;
 
 int gemm_i4g32_grouped(const GemmGroup *groups, int ngroups, int m_max, int N, int K, bool out_f32, hipStream_t st);
 bool gemm_skinny_ok(int H, int F);
