@@ -35,6 +35,10 @@ SIGNATURES = {
                                     c_void_p]),
     "chadq_attn_decode_mqa_workspace_floats": (c_size_t, [c_int, c_int, c_int]),
     "chadq_attn_decode_mqa": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "chadq_rope_table": (c_int, [c_void_p, c_int, c_int, c_float, c_void_p]),
+    "chadq_attn_decode_mqa_fused_workspace_floats": (c_size_t, [c_int, c_int, c_int]),
+    "chadq_attn_decode_mqa_fused": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                            c_void_p]),
     "chadq_geglu_bf16": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     "chadq_argmax_f32": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
 }

@@ -63,6 +63,9 @@ int rope_kv_launch(const float *, const int32_t *, float *, uint16_t *, uint16_t
 int attn_mqa_launch(const float *, const uint16_t *, const uint16_t *, const int32_t *, float *, uint16_t *, int, int, int,
                     hipStream_t);
 int geglu_launch(const float *, uint16_t *, int, hipStream_t);
+int rope_table_launch(float *, int, int, float, hipStream_t);
+int attn_mqa_fused_launch(const float *, const int32_t *, const float *, uint16_t *, uint16_t *, float *, uint16_t *, int, int, int,
+                          hipStream_t);
 int argmax_launch(const float *, int, float *, int32_t *, int32_t *, int32_t *, int, hipStream_t);
 
 }  // namespace chadq
@@ -253,6 +256,33 @@ int chadq_attn_decode_mqa(const float *q, const uint16_t *kcache_bf16, const uin
     CHADQ_REQUIRE(aligned16(kcache_bf16) && aligned16(q), CHADQ_ERR_ALIGN,
                   "chadq_attn_decode_mqa: q and kcache must be 16-byte aligned");
     return attn_mqa_launch(q, kcache_bf16, vcache_bf16, pos, workspace, out_bf16, hq, dh, max_ctx, st);
+}
+
+int chadq_rope_table(float *table, int dh, int max_ctx, float base, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(dh >= 2 && dh % 2 == 0 && max_ctx >= 1 && base > 0.f, CHADQ_ERR_SHAPE, "chadq_rope_table: dh=%d max_ctx=%d", dh,
+                  max_ctx);
+    CHADQ_REQUIRE(table, CHADQ_ERR_NULL, "chadq_rope_table: null pointer");
+    return rope_table_launch(table, dh, max_ctx, base, st);
+}
+
+size_t chadq_attn_decode_mqa_fused_workspace_floats(int hq, int dh, int max_ctx) {
+    if (hq < 1 || dh < 1 || max_ctx < 1) return 0;
+    return (size_t)((max_ctx + 31) / 32) * hq * (dh + 2);
+}
+
+int chadq_attn_decode_mqa_fused(const float *qkv, const int32_t *pos, const float *rope_table, uint16_t *kcache_bf16,
+                                uint16_t *vcache_bf16, float *workspace, uint16_t *out_bf16, int hq, int dh, int max_ctx,
+                                void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(hq >= 1 && hq <= 8 && dh >= 16 && dh <= 256 && dh % 16 == 0 && max_ctx >= 1 && max_ctx <= 65536, CHADQ_ERR_SHAPE,
+                  "chadq_attn_decode_mqa_fused: hq=%d dh=%d max_ctx=%d (hq <= 8, dh <= 256 and a multiple of 16, max_ctx <= 65536)",
+                  hq, dh, max_ctx);
+    CHADQ_REQUIRE(qkv && pos && rope_table && kcache_bf16 && vcache_bf16 && workspace && out_bf16, CHADQ_ERR_NULL,
+                  "chadq_attn_decode_mqa_fused: null pointer");
+    CHADQ_REQUIRE(aligned16(qkv) && aligned16(rope_table) && aligned16(kcache_bf16), CHADQ_ERR_ALIGN,
+                  "chadq_attn_decode_mqa_fused: qkv, rope_table and kcache must be 16-byte aligned");
+    return attn_mqa_fused_launch(qkv, pos, rope_table, kcache_bf16, vcache_bf16, workspace, out_bf16, hq, dh, max_ctx, st);
 }
 
 int chadq_geglu_bf16(const float *gu, uint16_t *h_bf16, int F, void *stream) {

@@ -236,14 +236,25 @@ __global__ __launch_bounds__(256) void attn_mqa_partial_kernel(const float *__re
     }
 }
 
-// out[h] = bf16( sum_b exp(m_b - M) * o_b / sum_b exp(m_b - M) * s_b ); one workgroup per head
+// out[h] = bf16( sum_b exp(m_b - M) * o_b / sum_b exp(m_b - M) * s_b ).  Workgroup (h, g): head h, columns
+// 64g..64g+63; its four waves take the slices b = w, w+4, ... so that all loads of a thread are independent and
+// in flight together, and meet in LDS.
 __global__ __launch_bounds__(256) void attn_mqa_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ pos,
                                                                uint16_t *__restrict__ out, int hq, int dh, int max_ctx) {
     const int ctx = min(max(pos[0], 0), max_ctx - 1) + 1, nb = (ctx + ATT_CS - 1) / ATT_CS, h = blockIdx.x, tid = threadIdx.x;
     __shared__ float s_f[ATT_MAX_NB];
     __shared__ float scratch[4];
+    __shared__ float s_num[4][64];
     const size_t stride = (size_t)hq * (dh + 2);
     const float *ph = part + (size_t)h * (dh + 2);
+    const int wave = tid >> 6, colw = blockIdx.y * 64 + (tid & 63), colc = colw < dh ? colw : dh - 1;
+    // the first 16 slices of this wave are requested before anything waits
+    float pre[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int b = wave + 4 * i;
+        pre[i] = ph[(size_t)(b < nb ? b : 0) * stride + 2 + colc];
+    }
     float m = -INFINITY;
     for (int b = tid; b < nb; b += 256) m = fmaxf(m, ph[b * stride]);
     const float M = block_max(m, scratch);
@@ -254,12 +265,202 @@ __global__ __launch_bounds__(256) void attn_mqa_combine_kernel(const float *__re
         den += f * ph[b * stride + 1];
     }
     den = block_sum(den, scratch);  // its barriers also publish s_f
-    if (tid < dh) {
-        float num = 0.f;
-#pragma unroll 8
-        for (int b = 0; b < nb; ++b) num += s_f[b] * ph[b * stride + 2 + tid];
-        out[(size_t)h * dh + tid] = (uint16_t)f32_to_bf16_bits(num / den);
+    float num = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int b = wave + 4 * i;
+        if (b < nb) num += s_f[b] * pre[i];
     }
+    for (int b = wave + 64; b < nb; b += 4) num += s_f[b] * ph[(size_t)b * stride + 2 + colc];
+    s_num[wave][tid & 63] = num;
+    __syncthreads();
+    if (tid < 64 && colw < dh) {
+        const float t = s_num[0][tid] + s_num[1][tid] + s_num[2][tid] + s_num[3][tid];
+        out[(size_t)h * dh + colw] = (uint16_t)f32_to_bf16_bits(t / den);
+    }
+}
+
+// ---- the same attention as one launch: RoPE, KV-cache write, split-context partials and their combination ----
+// table[p][j] = (cos, sin)(p * base^(-2j/dh)), p < max_ctx, j < dh/2; computed once per model.
+__global__ __launch_bounds__(256) void rope_table_kernel(float *__restrict__ table, int dh, int max_ctx, float base) {
+    const int half = dh / 2;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)max_ctx * half) return;
+    const int p = (int)(i / half), j = (int)(i % half);
+    const float inv = powf(base, -2.f * (float)j / (float)dh);
+    float sn, cs;
+    sincosf((float)p * inv, &sn, &cs);
+    table[2 * i] = cs;
+    table[2 * i + 1] = sn;
+}
+
+// Sum over each 32-lane half of the wave; valid in lanes 16..31 and 48..63 (data-parallel primitives only: a
+// cross-lane read through LDS costs a wait each, and there are 160 of these reductions per workgroup).
+__device__ __forceinline__ float half_wave_sum_hi(float v) {
+    v += dpp_f32<0x128, 0xF>(v);  // row_ror:8
+    v += dpp_f32<0x124, 0xF>(v);  // row_ror:4
+    v += dpp_f32<0x122, 0xF>(v);  // row_ror:2
+    v += dpp_f32<0x121, 0xF>(v);  // row_ror:1: every lane of a 16-lane row holds the row sum
+    v += dpp_f32<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
+    return v;
+}
+
+// Workgroup b: positions [32b, 32b+32).  qkv fp32 = [hq*dh | dh | dh] straight from the projection.  Every
+// workgroup rotates q itself (table lookup); the one that owns position pos also rotates k, writes row pos of both
+// caches and uses the new row from registers/LDS instead of reading it back.  Partials as attn_mqa_partial_kernel;
+// attn_mqa_combine_kernel follows.  (Letting the last workgroup to finish do the combination in the same launch
+// was tried and lost: one workgroup pulling every partial through one CU took longer than a second launch.)
+__global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__restrict__ qkv, const int32_t *__restrict__ pos,
+                                                             const float *__restrict__ table, uint16_t *__restrict__ kc,
+                                                             uint16_t *__restrict__ vc, float *__restrict__ ws,
+                                                             uint16_t *__restrict__ out, int hq, int dh, int max_ctx) {
+    const int p = min(max(pos[0], 0), max_ctx - 1), ctx = p + 1;
+    const int p0 = blockIdx.x * ATT_CS;
+    if (p0 >= ctx) return;
+    const bool own = (p - p0) < ATT_CS;  // this slice contains the new position
+    float *part = ws;
+    __shared__ __attribute__((aligned(16))) float s_sc[8][ATT_CS];  // scores, then probabilities
+    __shared__ __attribute__((aligned(16))) uint16_t s_krow[256];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int half = dh >> 1, hw = lane >> 5, c = lane & 31, lpr = dh >> 3;
+
+    // V: thread t owns column t of every row of the slice
+    const int col = tid < dh ? tid : dh - 1;
+    uint16_t vv[ATT_CS];
+#pragma unroll
+    for (int i = 0; i < ATT_CS; ++i) {
+        const int pi = (p0 + i < ctx) ? p0 + i : ctx - 1;
+        vv[i] = vc[(size_t)pi * dh + col];
+    }
+    // K: wave w owns rows 8w..8w+7 of the slice, two rows per load instruction
+    const int cc = c < lpr ? c : 0;
+    u32x4 kv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int pl = wave * 8 + 2 * i + hw;
+        const int pi = (p0 + pl < ctx) ? p0 + pl : ctx - 1;
+        kv[i] = *reinterpret_cast<const u32x4 *>(kc + (size_t)pi * dh + cc * 8);
+    }
+    // q: the lane's 8 columns of every head, the 8 columns they rotate with, and the angles
+    const int colq = cc * 8, lo = colq < half;
+    const int colp = lo ? colq + half : colq - half;  // partner columns
+    const int jt = lo ? colq : colq - half;           // rotation index of element 0
+    f32x4 qa[8], qb[8], pa[8], pb[8];
+#pragma unroll
+    for (int h = 0; h < 8; ++h) {
+        const float *qh = qkv + (size_t)(h < hq ? h : 0) * dh;
+        qa[h] = *reinterpret_cast<const f32x4 *>(qh + colq);
+        qb[h] = *reinterpret_cast<const f32x4 *>(qh + colq + 4);
+        pa[h] = *reinterpret_cast<const f32x4 *>(qh + colp);
+        pb[h] = *reinterpret_cast<const f32x4 *>(qh + colp + 4);
+    }
+    const float *tp = table + ((size_t)p * half + jt) * 2;
+    f32x4 t0 = *reinterpret_cast<const f32x4 *>(tp), t1 = *reinterpret_cast<const f32x4 *>(tp + 4),
+          t2 = *reinterpret_cast<const f32x4 *>(tp + 8), t3 = *reinterpret_cast<const f32x4 *>(tp + 12);
+    // the owner's new K/V row
+    float ka = 0.f, kb = 0.f, kcs = 1.f, ksn = 0.f, vnew = 0.f;
+    if (own) {
+        if (tid < half) {
+            ka = qkv[(size_t)hq * dh + tid];
+            kb = qkv[(size_t)hq * dh + tid + half];
+            kcs = table[((size_t)p * half + tid) * 2];
+            ksn = table[((size_t)p * half + tid) * 2 + 1];
+        }
+        if (tid < dh) vnew = qkv[(size_t)(hq + 1) * dh + tid];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    if (own) {
+        if (tid < half) {
+            const uint16_t ra = (uint16_t)f32_to_bf16_bits(ka * kcs - kb * ksn), rb = (uint16_t)f32_to_bf16_bits(kb * kcs + ka * ksn);
+            s_krow[tid] = ra;
+            s_krow[tid + half] = rb;
+            kc[(size_t)p * dh + tid] = ra;
+            kc[(size_t)p * dh + tid + half] = rb;
+        }
+        const uint16_t vb16 = (uint16_t)f32_to_bf16_bits(vnew);
+        if (tid < dh) vc[(size_t)p * dh + tid] = vb16;
+#pragma unroll
+        for (int i = 0; i < ATT_CS; ++i)
+            if (p0 + i == p) vv[i] = vb16;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (p0 + wave * 8 + 2 * i + hw == p) kv[i] = *reinterpret_cast<const u32x4 *>(s_krow + cc * 8);
+    }
+
+    // rotate q: low columns a*cos - b*sin, high columns b*cos + a*sin, (a, b) = (low, high) element of the pair
+    {
+        const float cs[8] = {t0.x, t0.z, t1.x, t1.z, t2.x, t2.z, t3.x, t3.z};
+        const float sn[8] = {t0.y, t0.w, t1.y, t1.w, t2.y, t2.w, t3.y, t3.w};
+        const float sg = lo ? -1.f : 1.f;
+#pragma unroll
+        for (int h = 0; h < 8; ++h) {
+            const float own8[8] = {qa[h].x, qa[h].y, qa[h].z, qa[h].w, qb[h].x, qb[h].y, qb[h].z, qb[h].w};
+            const float par8[8] = {pa[h].x, pa[h].y, pa[h].z, pa[h].w, pb[h].x, pb[h].y, pb[h].z, pb[h].w};
+            float r[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) r[e] = own8[e] * cs[e] + sg * par8[e] * sn[e];
+            qa[h] = f32x4{r[0], r[1], r[2], r[3]};
+            qb[h] = f32x4{r[4], r[5], r[6], r[7]};
+        }
+    }
+
+    const bool live = c < lpr;
+    const float scale = rsqrtf((float)dh);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int pl = wave * 8 + 2 * i + hw;
+        const uint32_t kk[4] = {kv[i].x, kv[i].y, kv[i].z, kv[i].w};
+        float k8[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            k8[2 * e] = live ? bf16_bits_to_f32(kk[e] & 0xFFFFu) : 0.f;
+            k8[2 * e + 1] = live ? bf16_bits_to_f32(kk[e] >> 16) : 0.f;
+        }
+#pragma unroll
+        for (int h = 0; h < 8; ++h) {
+            float acc = qa[h].x * k8[0] + qa[h].y * k8[1] + qa[h].z * k8[2] + qa[h].w * k8[3] + qb[h].x * k8[4] +
+                        qb[h].y * k8[5] + qb[h].z * k8[6] + qb[h].w * k8[7];
+            acc = half_wave_sum_hi(acc);
+            if (c == 16) s_sc[h][pl] = (p0 + pl < ctx && h < hq) ? acc * scale : -INFINITY;
+        }
+    }
+    __syncthreads();
+    {
+        // softmax of the slice: thread -> (head tid/32, position tid%32)
+        const int h = tid >> 5, i = tid & 31;
+        const float s = s_sc[h][i];
+        float mx = s;
+        for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        const float pr = (h < hq) ? __expf(s - mx) : 0.f;
+        float sum = pr;
+        for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+        s_sc[h][i] = pr;
+        if (i == 0 && h < hq) {
+            float *dst = part + ((size_t)blockIdx.x * hq + h) * (dh + 2);
+            dst[0] = mx;
+            dst[1] = sum;
+        }
+    }
+    __syncthreads();
+    float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < ATT_CS; i += 4) {
+        const float v0 = bf16_bits_to_f32(vv[i]), v1 = bf16_bits_to_f32(vv[i + 1]), v2 = bf16_bits_to_f32(vv[i + 2]),
+                    v3 = bf16_bits_to_f32(vv[i + 3]);
+#pragma unroll
+        for (int h = 0; h < 8; ++h) {
+            const f32x4 p4 = *reinterpret_cast<const f32x4 *>(&s_sc[h][i]);
+            o[h] += p4.x * v0 + p4.y * v1 + p4.z * v2 + p4.w * v3;
+        }
+    }
+    if (tid < dh) {
+#pragma unroll
+        for (int h = 0; h < 8; ++h)
+            if (h < hq) part[((size_t)blockIdx.x * hq + h) * (dh + 2) + 2 + tid] = o[h];
+    }
+
 }
 
 // h = bf16( gelu_tanh(g) * u ), gu = [g(F) | u(F)] fp32
@@ -377,8 +578,22 @@ int attn_mqa_launch(const float *q, const uint16_t *kc, const uint16_t *vc, cons
                     int hq, int dh, int max_ctx, hipStream_t st) {
     const int nb = (max_ctx + ATT_CS - 1) / ATT_CS;
     hipLaunchKernelGGL(attn_mqa_partial_kernel, dim3(nb), dim3(256), 0, st, q, kc, vc, pos, part, hq, dh, max_ctx);
-    hipLaunchKernelGGL(attn_mqa_combine_kernel, dim3(hq), dim3(256), 0, st, part, pos, out, hq, dh, max_ctx);
+    hipLaunchKernelGGL(attn_mqa_combine_kernel, dim3(hq, (dh + 63) / 64), dim3(256), 0, st, part, pos, out, hq, dh, max_ctx);
     return hip_check(hipGetLastError(), "attn_mqa launch");
+}
+
+int rope_table_launch(float *table, int dh, int max_ctx, float base, hipStream_t st) {
+    const int64_t n = (int64_t)max_ctx * (dh / 2);
+    hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, table, dh, max_ctx, base);
+    return hip_check(hipGetLastError(), "rope_table launch");
+}
+
+int attn_mqa_fused_launch(const float *qkv, const int32_t *pos, const float *table, uint16_t *kc, uint16_t *vc, float *ws,
+                          uint16_t *out, int hq, int dh, int max_ctx, hipStream_t st) {
+    const int nb = (max_ctx + ATT_CS - 1) / ATT_CS;
+    hipLaunchKernelGGL(attn_mqa_fused_kernel, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, out, hq, dh, max_ctx);
+    hipLaunchKernelGGL(attn_mqa_combine_kernel, dim3(hq, (dh + 63) / 64), dim3(256), 0, st, ws, pos, out, hq, dh, max_ctx);
+    return hip_check(hipGetLastError(), "attn_mqa_fused launch");
 }
 
 int geglu_launch(const float *gu, uint16_t *h, int F, hipStream_t st) {

@@ -73,7 +73,15 @@ class QuantDecoder:
         self.ksplit = next((s for s in (4, 2) if c.ffn % (s * 4096) == 0), 1)
         self.gu, self.h, self.dn = z(2 * c.ffn, f32), z(c.ffn, bf16), z(self.ksplit * c.d, f32)
         self.logits = z(c.vocab, f32)
-        self.part = z(self.lib.chadq_attn_decode_mqa_workspace_floats(c.hq, c.dh, c.max_ctx), f32)
+        # attention with the rotation and the cache write folded in, where its limits allow
+        self.fused_attn = c.dh % 16 == 0 and c.max_ctx <= 65536
+        if self.fused_attn:
+            self.part = z(self.lib.chadq_attn_decode_mqa_fused_workspace_floats(c.hq, c.dh, c.max_ctx), f32)
+            self.rope = z(c.max_ctx * c.dh, f32)
+            _lib.check(self.lib.chadq_rope_table(self.rope.data_ptr(), c.dh, c.max_ctx, c.rope_base,
+                                                 torch.cuda.current_stream().cuda_stream), "chadq_rope_table")
+        else:
+            self.part = z(self.lib.chadq_attn_decode_mqa_workspace_floats(c.hq, c.dh, c.max_ctx), f32)
         self.scratch = z(512, f32)
         self.token, self.pos = z(1, i32), z(1, i32)
         self.kcache = [z(c.max_ctx * c.dh, bf16) for _ in range(c.n_layers)]
@@ -103,12 +111,18 @@ class QuantDecoder:
         for li, L in enumerate(self.w["layers"]):
             self._norm(pending, L["ln1"])
             self._gemv(self.xn, L["wqkv"], self.qkv)
-            _lib.check(lib.chadq_rope_kv_write(self.qkv.data_ptr(), self.pos.data_ptr(), self.q.data_ptr(),
-                                               self.kcache[li].data_ptr(), self.vcache[li].data_ptr(), c.hq, c.dh,
-                                               c.max_ctx, c.rope_base, s), "chadq_rope_kv_write")
-            _lib.check(lib.chadq_attn_decode_mqa(self.q.data_ptr(), self.kcache[li].data_ptr(), self.vcache[li].data_ptr(),
-                                                 self.pos.data_ptr(), self.part.data_ptr(), self.att.data_ptr(), c.hq, c.dh,
-                                                 c.max_ctx, s), "chadq_attn_decode_mqa")
+            if self.fused_attn:
+                _lib.check(lib.chadq_attn_decode_mqa_fused(self.qkv.data_ptr(), self.pos.data_ptr(), self.rope.data_ptr(),
+                                                           self.kcache[li].data_ptr(), self.vcache[li].data_ptr(),
+                                                           self.part.data_ptr(), self.att.data_ptr(), c.hq, c.dh, c.max_ctx, s),
+                           "chadq_attn_decode_mqa_fused")
+            else:
+                _lib.check(lib.chadq_rope_kv_write(self.qkv.data_ptr(), self.pos.data_ptr(), self.q.data_ptr(),
+                                                   self.kcache[li].data_ptr(), self.vcache[li].data_ptr(), c.hq, c.dh,
+                                                   c.max_ctx, c.rope_base, s), "chadq_rope_kv_write")
+                _lib.check(lib.chadq_attn_decode_mqa(self.q.data_ptr(), self.kcache[li].data_ptr(), self.vcache[li].data_ptr(),
+                                                     self.pos.data_ptr(), self.part.data_ptr(), self.att.data_ptr(), c.hq, c.dh,
+                                                     c.max_ctx, s), "chadq_attn_decode_mqa")
             self._gemv(self.att, L["wo"], self.ao)
             self._norm(self.ao, L["ln2"])
             self._gemv(self.xn, L["wgu"], self.gu)

@@ -172,6 +172,22 @@ size_t chadq_attn_decode_mqa_workspace_floats(int hq, int dh, int max_ctx);
 int chadq_attn_decode_mqa(const float *q, const uint16_t *kcache_bf16, const uint16_t *vcache_bf16, const int32_t *pos,
                           float *workspace, uint16_t *out_bf16, int hq, int dh, int max_ctx, void *stream);
 
+/* table fp32 [max_ctx, dh/2, 2] = (cos, sin) of p * base^(-2j/dh): the rotation angles chadq_rope_kv_write computes. */
+int chadq_rope_table(float *table, int dh, int max_ctx, float base, void *stream);
+
+/* Floats of workspace chadq_attn_decode_mqa_fused needs. */
+size_t chadq_attn_decode_mqa_fused_workspace_floats(int hq, int dh, int max_ctx);
+
+/*
+ * chadq_rope_kv_write and chadq_attn_decode_mqa with the rotation and the cache write folded into the attention
+ * kernel: rotates q and k of qkv (angles from rope_table), writes row pos[0] of both caches, attends over rows
+ * 0..pos[0] and writes out bf16 [hq*dh].  qkv fp32 = [hq*dh | dh | dh].
+ * hq <= 8, dh <= 256 and a multiple of 16, max_ctx <= 65536; qkv, rope_table and kcache 16-byte aligned.
+ */
+int chadq_attn_decode_mqa_fused(const float *qkv, const int32_t *pos, const float *rope_table, uint16_t *kcache_bf16,
+                                uint16_t *vcache_bf16, float *workspace, uint16_t *out_bf16, int hq, int dh, int max_ctx,
+                                void *stream);
+
 /* h[F] = bf16( gelu_tanh(gu[i]) * gu[F+i] ). */
 int chadq_geglu_bf16(const float *gu, uint16_t *h_bf16, int F, void *stream);
 

@@ -161,6 +161,50 @@ def test_attn_decode_mqa(lib, hq, dh, pos, max_ctx):
     assert O.rel_l2(O.bf16_to_f32(bits(out)).reshape(hq, dh), want) < 1e-2
 
 
+@pytest.mark.parametrize("hq,dh,pos,max_ctx", [(8, 256, 0, 64), (8, 256, 31, 64), (8, 256, 32, 4096), (8, 256, 2047, 4096),
+                                               (8, 256, 4095, 4096), (8, 256, 8191, 8192), (3, 64, 200, 300), (1, 16, 70, 128)])
+def test_attn_decode_mqa_fused_equals_rope_write_attend(lib, hq, dh, pos, max_ctx):
+    r = rng(7 * hq + dh + pos)
+    qkv = r.standard_normal((hq + 2) * dh).astype(np.float32)
+    kc = O.f32_to_bf16(r.standard_normal((max_ctx, dh)).astype(np.float32))
+    vc = O.f32_to_bf16(r.standard_normal((max_ctx, dh)).astype(np.float32))
+    tq, tk, tv = dev(qkv), bf16_tensor(kc.reshape(-1)), bf16_tensor(vc.reshape(-1))
+    tp = torch.tensor([pos], dtype=torch.int32, device=DEV)
+    table = torch.zeros(max_ctx * dh, dtype=torch.float32, device=DEV)
+    chk(lib.chadq_rope_table(table.data_ptr(), dh, max_ctx, 10000.0, stream()), "table")
+    ws = torch.zeros(lib.chadq_attn_decode_mqa_fused_workspace_floats(hq, dh, max_ctx), dtype=torch.float32, device=DEV)
+    out = torch.zeros(hq * dh, dtype=torch.bfloat16, device=DEV)
+    # oracle: rotate, write the cache row, attend
+    q = O.rope_rotate_half(qkv[: hq * dh].reshape(hq, dh), pos)
+    kc[pos] = O.f32_to_bf16(O.rope_rotate_half(qkv[hq * dh: (hq + 1) * dh], pos))
+    vc[pos] = O.f32_to_bf16(qkv[(hq + 1) * dh:])
+    kk = O.bf16_to_f32(kc[: pos + 1]).astype(np.float64)
+    vv = O.bf16_to_f32(vc[: pos + 1]).astype(np.float64)
+    s = q.astype(np.float64) @ kk.T / np.sqrt(dh)
+    pr = np.exp(s - s.max(-1, keepdims=True))
+    want = (pr / pr.sum(-1, keepdims=True)) @ vv
+    for call in range(2):  # the second call finds the new row already in the cache
+        chk(lib.chadq_attn_decode_mqa_fused(tq.data_ptr(), tp.data_ptr(), table.data_ptr(), tk.data_ptr(), tv.data_ptr(),
+                                            ws.data_ptr(), out.data_ptr(), hq, dh, max_ctx, stream()), "attn fused")
+        torch.cuda.synchronize()
+        assert O.rel_l2(O.bf16_to_f32(bits(out)).reshape(hq, dh), want) < 1e-2, "call %d" % call
+    kb, vb = bits(tk).reshape(max_ctx, dh), bits(tv).reshape(max_ctx, dh)
+    assert np.array_equal(vb, vc)  # V row written exactly, every other row untouched
+    assert np.abs(O.bf16_to_f32(kb[pos]) - O.bf16_to_f32(kc[pos])).max() < 4e-2  # fp32 sin/cos of large angles
+    rest = np.ones(max_ctx, bool)
+    rest[pos] = False
+    assert np.array_equal(kb[rest], kc[rest])
+
+
+def test_rope_table_matches_the_rotation(lib):
+    dh, ctx = 64, 300
+    table = torch.zeros(ctx * dh, dtype=torch.float32, device=DEV)
+    chk(lib.chadq_rope_table(table.data_ptr(), dh, ctx, 10000.0, stream()), "table")
+    t = table.cpu().numpy().reshape(ctx, dh // 2, 2)
+    ang = np.arange(ctx)[:, None] * (10000.0 ** (-2.0 * np.arange(dh // 2) / dh))[None, :]
+    assert np.abs(t[..., 0] - np.cos(ang)).max() < 2e-4 and np.abs(t[..., 1] - np.sin(ang)).max() < 2e-4
+
+
 @pytest.mark.parametrize("F", [1, 255, 16384])
 def test_geglu(lib, F):
     gu = (rng(F).standard_normal(2 * F) * 3).astype(np.float32)
