@@ -22,6 +22,7 @@ SIGNATURES = {
     "chadq_dequant_i8row": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "chadq_gemv_i4g32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "chadq_gemv_i4g32_splitk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "chadq_gemv_i4g32_splitk_geglu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "chadq_gemv_i8row": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "chadq_gemm_i4g32_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "chadq_gemm_i8row_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),

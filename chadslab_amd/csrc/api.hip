@@ -59,6 +59,7 @@ int moe_ffn_i4g32_launch(const uint16_t *, const float *, const chadq_moe_expert
 int embed_launch(const int32_t *, const uint8_t *, const uint16_t *, float *, int, int, hipStream_t);
 int add_rmsnorm_launch(float *, const float *, int, const float *, uint16_t *, int, float, hipStream_t);
 int gemv_i4g32_splitk_launch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
+int gemv_i4g32_splitk_geglu_launch(const float *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
 int rope_kv_launch(const float *, const int32_t *, float *, uint16_t *, uint16_t *, int, int, int, float, hipStream_t);
 int attn_mqa_launch(const float *, const uint16_t *, const uint16_t *, const int32_t *, float *, uint16_t *, int, int, int,
                     hipStream_t);
@@ -143,6 +144,19 @@ int chadq_gemv_i4g32_splitk(const uint16_t *x_bf16, const uint8_t *wp, const uin
     CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(wp) && aligned16(scale_f16), CHADQ_ERR_ALIGN,
                   "chadq_gemv_i4g32_splitk: x, wp and scale must be 16-byte aligned");
     return gemv_i4g32_splitk_launch(x_bf16, wp, scale_f16, y_parts, N, K, ksplit, st);
+}
+
+int chadq_gemv_i4g32_splitk_geglu(const float *gu, const uint8_t *wp, const uint16_t *scale_f16, float *y_parts, int N, int K,
+                                  int ksplit, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(N >= 1 && K >= 4096 && ksplit >= 1 && ksplit <= 64 && K % (ksplit * 4096) == 0, CHADQ_ERR_SHAPE,
+                  "chadq_gemv_i4g32_splitk_geglu: N=%d K=%d ksplit=%d (K must be a multiple of ksplit*4096)", N, K, ksplit);
+    CHADQ_REQUIRE((int64_t)N * (K / 2) < ((int64_t)1 << 31), CHADQ_ERR_SHAPE,
+                  "chadq_gemv_i4g32_splitk_geglu: N*K/2 = %lld bytes exceeds 2^31", (long long)N * (K / 2));
+    CHADQ_REQUIRE(gu && wp && scale_f16 && y_parts, CHADQ_ERR_NULL, "chadq_gemv_i4g32_splitk_geglu: null pointer");
+    CHADQ_REQUIRE(aligned16(gu) && aligned16(wp) && aligned16(scale_f16), CHADQ_ERR_ALIGN,
+                  "chadq_gemv_i4g32_splitk_geglu: gu, wp and scale must be 16-byte aligned");
+    return gemv_i4g32_splitk_geglu_launch(gu, wp, scale_f16, y_parts, N, K, ksplit, st);
 }
 
 int chadq_gemv_i8row(const float *x, const int8_t *w8, const float *scale, float *y, int M, int N, int K,

@@ -154,6 +154,13 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
     return __builtin_amdgcn_fdot2_f32_bf16(as_bf16x2(a), as_bf16x2(b), c, false);
 }
 
+// GELU, tanh form: 0.5 g (1 + tanh z), z = sqrt(2/pi) (g + 0.044715 g^3), which equals g / (1 + exp(-2z)).
+// One exp and one reciprocal: cheap enough to be recomputed by every workgroup that stages an activation vector.
+__device__ __forceinline__ float gelu_tanh_dev(float g) {
+    const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    return g * __builtin_amdgcn_rcpf(1.f + __expf(-2.f * z));
+}
+
 // data-parallel-primitive move: value of `v` from the lane selected by CTRL, 0 where masked off
 template <int CTRL, int ROW_MASK>
 __device__ __forceinline__ float dpp_f32(float v) {

@@ -467,9 +467,7 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
 __global__ __launch_bounds__(256) void geglu_kernel(const float *__restrict__ gu, uint16_t *__restrict__ h, int F) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < F) {
-        const float g = gu[i], u = gu[F + i];
-        const float t = tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g));
-        h[i] = (uint16_t)f32_to_bf16_bits(0.5f * g * (1.f + t) * u);
+        h[i] = (uint16_t)f32_to_bf16_bits(gelu_tanh_dev(gu[i]) * gu[F + i]);
     }
 }
 

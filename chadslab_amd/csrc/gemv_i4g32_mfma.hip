@@ -65,7 +65,9 @@ struct GemvCfg {
 };
 
 // waves_per_eu(4): at most 128 VGPRs, which also makes the compiler pick the MFMA form that writes VGPRs.
-template <int MT, int HP, int S, int RBW, int D, int KC>
+// XG: the activation vector is not given but formed while staging: x[k] = bf16( gelu_tanh(gu[k]) * gu[K + k] ) from
+// gu fp32 [2K] (`x` then points at gu) - the GeGLU of a gated FFN folded into its down projection.  M = 1 only.
+template <int MT, int HP, int S, int RBW, int D, int KC, bool XG = false>
 __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) void gemv_i4g32_mfma_kernel(
     const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
     float *__restrict__ y, int N, int K, int kspan) {
@@ -115,6 +117,7 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
     for (int kc0 = kbeg; kc0 < kend; kc0 += KC) {
         // 1. activation loads FIRST.  Piece `it` = tid + T*q of pass p: row m = it / 512, i8 = it % 512.
         u32x4 xr[MP][XI];
+        f32x4 gr[XG ? XI : 1][4];  // XG: 8 gate and 8 up values per piece
 #pragma unroll
         for (int p = 0; p < MP; ++p)
 #pragma unroll
@@ -122,7 +125,15 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
                 const int m = (T * q) / (KC / 8);  // same for the whole workgroup: T divides KC/8
                 if (m >= MPASS || p * MPASS + m >= M) continue;  // compile time after unrolling
                 const int k = kc0 + 8 * ((tid + T * q) % (KC / 8));
-                xr[p][q] = *reinterpret_cast<const u32x4 *>(x + (k < K ? (size_t)(p * MPASS + m) * K + k : 0));
+                if constexpr (XG) {
+                    const float *gp = reinterpret_cast<const float *>(x) + (k < K ? k : 0);
+                    gr[q][0] = *reinterpret_cast<const f32x4 *>(gp);
+                    gr[q][1] = *reinterpret_cast<const f32x4 *>(gp + 4);
+                    gr[q][2] = *reinterpret_cast<const f32x4 *>(gp + K);
+                    gr[q][3] = *reinterpret_cast<const f32x4 *>(gp + K + 4);
+                } else {
+                    xr[p][q] = *reinterpret_cast<const u32x4 *>(x + (k < K ? (size_t)(p * MPASS + m) * K + k : 0));
+                }
             }
 
         // 2. the wave's scale tile in one load.  Needs G % 8 == 0 (16-byte aligned pieces), checked on the host.
@@ -153,7 +164,19 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
                 const int m = (T * q) / (KC / 8);
                 if (m >= MPASS || p * MPASS + m >= M) continue;  // padding row: its A lanes read the zero block
                 const int i8 = (tid + T * q) % (KC / 8);
-                u32x4 v = xr[p][q];
+                u32x4 v;
+                if constexpr (XG) {
+                    const float g8[8] = {gr[q][0].x, gr[q][0].y, gr[q][0].z, gr[q][0].w, gr[q][1].x, gr[q][1].y, gr[q][1].z, gr[q][1].w};
+                    const float u8[8] = {gr[q][2].x, gr[q][2].y, gr[q][2].z, gr[q][2].w, gr[q][3].x, gr[q][3].y, gr[q][3].z, gr[q][3].w};
+                    uint32_t hb[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        hb[e] = f32_to_bf16_bits(gelu_tanh_dev(g8[e]) * u8[e]);
+                    }
+                    v = u32x4{hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16), hb[4] | (hb[5] << 16), hb[6] | (hb[7] << 16)};
+                } else {
+                    v = xr[p][q];
+                }
                 if (kc0 + 8 * i8 >= K) v = u32x4{0, 0, 0, 0};
                 uint32_t a[4] = {v.x, v.y, v.z, v.w}, o[4];
                 float sum = 0.f;
@@ -242,18 +265,18 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
 
 int gemv_i4g32_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
 
-template <int MT, int HP, int S, int RBW, int D, int KC = 4096>
+template <int MT, int HP, int S, int RBW, int D, int KC = 4096, bool XG = false>
 static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K,
                        hipStream_t st, int ksplit = 1) {
     typedef GemvCfg<MT, HP, S, RBW, KC> C;
     static bool attr_set = false;
     if (!attr_set) {
-        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC>),
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XG>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::TOTAL));
         attr_set = true;
     }
     const int units = (N + C::UR - 1) / C::UR;
-    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC>), dim3((units + RBW - 1) / RBW, ksplit), dim3(256 * RBW),
+    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XG>), dim3((units + RBW - 1) / RBW, ksplit), dim3(256 * RBW),
                        C::TOTAL, st, x, wp, sc, y, N, K, K / ksplit);
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma launch");
 }
@@ -294,6 +317,12 @@ int gemv_i4g32_mfma_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_
 int gemv_i4g32_splitk_launch(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y_parts, int N, int K,
                              int ksplit, hipStream_t st) {
     return launch_mfma<1, 4, 8, 1, 3>(x, wp, sc, y_parts, N, K, st, ksplit);
+}
+
+// The same with x[k] = bf16( gelu_tanh(gu[k]) * gu[K + k] ) formed inside the kernel.
+int gemv_i4g32_splitk_geglu_launch(const float *gu, const uint8_t *wp, const uint16_t *sc, float *y_parts, int N, int K,
+                                   int ksplit, hipStream_t st) {
+    return launch_mfma<1, 4, 8, 1, 3, 4096, true>(reinterpret_cast<const uint16_t *>(gu), wp, sc, y_parts, N, K, st, ksplit);
 }
 
 }  // namespace chadq

@@ -126,12 +126,12 @@ class QuantDecoder:
             self._gemv(self.att, L["wo"], self.ao)
             self._norm(self.ao, L["ln2"])
             self._gemv(self.xn, L["wgu"], self.gu)
-            _lib.check(lib.chadq_geglu_bf16(self.gu.data_ptr(), self.h.data_ptr(), c.ffn, s), "chadq_geglu_bf16")
-            if self.ksplit > 1:
-                _lib.check(lib.chadq_gemv_i4g32_splitk(self.h.data_ptr(), L["wd"].packed.data_ptr(), L["wd"].scale.data_ptr(),
-                                                       self.dn.data_ptr(), c.d, c.ffn, self.ksplit, s),
-                           "chadq_gemv_i4g32_splitk")
+            if self.ksplit > 1:  # GeGLU folded into the split-K down projection
+                _lib.check(lib.chadq_gemv_i4g32_splitk_geglu(self.gu.data_ptr(), L["wd"].packed.data_ptr(),
+                                                             L["wd"].scale.data_ptr(), self.dn.data_ptr(), c.d, c.ffn,
+                                                             self.ksplit, s), "chadq_gemv_i4g32_splitk_geglu")
             else:
+                _lib.check(lib.chadq_geglu_bf16(self.gu.data_ptr(), self.h.data_ptr(), c.ffn, s), "chadq_geglu_bf16")
                 self._gemv(self.h, L["wd"], self.dn)
             pending = self.dn
         self._norm(pending, self.w["lnf"])

@@ -90,6 +90,13 @@ int chadq_gemv_i4g32_splitk(const uint16_t *x_bf16, const uint8_t *wp, const uin
                             int K, int ksplit, void *stream);
 
 /*
+ * chadq_gemv_i4g32_splitk with the GeGLU of a gated FFN folded in: the activation is formed inside the kernel as
+ * x[k] = bf16( gelu_tanh(gu[k]) * gu[K + k] ) from gu fp32 [2K] (what chadq_geglu_bf16 would write).  gu 16-byte aligned.
+ */
+int chadq_gemv_i4g32_splitk_geglu(const float *gu, const uint8_t *wp, const uint16_t *scale_f16, float *y_parts, int N, int K,
+                                  int ksplit, void *stream);
+
+/*
  * y[m,n] = scale[n] * sum_k x[m,k] * W[n,k]                                 (config 0)
  * x fp32 [M,K], W int8 [N,K], scale fp32 [N], y fp32 [M,N], 1 <= M <= 16, K % 16 == 0.
  */

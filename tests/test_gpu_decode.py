@@ -102,6 +102,29 @@ def test_gemv_splitk_parts(lib, n, k, ksplit):
         chk(lib.chadq_gemv_i4g32_splitk(tx.data_ptr(), tp_.data_ptr(), ts.data_ptr(), parts.data_ptr(), n, k, 3, stream()), "splitk")
 
 
+@pytest.mark.parametrize("n,k,ksplit", [(2048, 16384, 4), (100, 8192, 1)])
+def test_gemv_splitk_geglu_equals_geglu_then_gemv(lib, n, k, ksplit):
+    r = rng(3 * n + k + ksplit)
+    u = r.integers(0, 16, (n, k), dtype=np.uint8)
+    packed = (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8)
+    s = r.lognormal(-5, 0.5, (n, k // 32)).astype(np.float16)
+    gu = (r.standard_normal(2 * k) * 2).astype(np.float32)
+    tp_, ts, tg = dev(packed), dev(s), dev(gu)
+    parts = torch.zeros(ksplit * n, dtype=torch.float32, device=DEV)
+    chk(lib.chadq_gemv_i4g32_splitk_geglu(tg.data_ptr(), tp_.data_ptr(), ts.data_ptr(), parts.data_ptr(), n, k, ksplit, stream()),
+        "splitk geglu")
+    # the unfused pair on the GPU must give the same bits: same GeGLU formula, same GEMV kernel
+    h = torch.zeros(k, dtype=torch.bfloat16, device=DEV)
+    parts2 = torch.zeros(ksplit * n, dtype=torch.float32, device=DEV)
+    chk(lib.chadq_geglu_bf16(tg.data_ptr(), h.data_ptr(), k, stream()), "geglu")
+    chk(lib.chadq_gemv_i4g32_splitk(h.data_ptr(), tp_.data_ptr(), ts.data_ptr(), parts2.data_ptr(), n, k, ksplit, stream()), "splitk")
+    assert torch.equal(parts, parts2)
+    # and the oracle
+    hb = O.f32_to_bf16(O.gelu_tanh(gu[:k]) * gu[k:])[None, :]
+    want = O.qgemm_int4g32_f64(hb, packed, s)[0]
+    assert O.rel_l2(parts.cpu().numpy().reshape(ksplit, n).sum(0), want) < 2e-3
+
+
 @pytest.mark.parametrize("hq,dh,pos", [(8, 256, 0), (8, 256, 2047), (4, 64, 100), (1, 8, 3)])
 def test_rope_kv_write(lib, hq, dh, pos):
     r = rng(hq * 1000 + dh + pos)
