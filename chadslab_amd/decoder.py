@@ -57,6 +57,29 @@ def random_weights(cfg: DecoderConfig, seed: int, device) -> Dict:
     return {"layers": layers, "lnf": norm(), "emb": q(cfg.vocab, cfg.d)}
 
 
+def save_weights(path: str, cfg: DecoderConfig, weights: Dict) -> None:
+    """Writes a decoder's weights and configuration to one weight-container file (chadslab_amd.wfile)."""
+    from dataclasses import asdict
+
+    from . import wfile
+
+    flat = {"lnf": weights["lnf"], "emb": weights["emb"]}
+    for li, L in enumerate(weights["layers"]):
+        for k, v in L.items():
+            flat["layers.%d.%s" % (li, k)] = v
+    wfile.save(path, flat, meta={"decoder_config": asdict(cfg)})
+
+
+def load_weights(path: str, device):
+    """Inverse of save_weights: returns (DecoderConfig, weights) with every tensor on `device`."""
+    from . import wfile
+
+    cfg = DecoderConfig(**wfile.read_header(path)["meta"]["decoder_config"])
+    flat = wfile.load(path, device)
+    layers = [{k: flat["layers.%d.%s" % (li, k)] for k in ("ln1", "wqkv", "wo", "ln2", "wgu", "wd")} for li in range(cfg.n_layers)]
+    return cfg, {"layers": layers, "lnf": flat["lnf"], "emb": flat["emb"]}
+
+
 class QuantDecoder:
     def __init__(self, cfg: DecoderConfig, weights: Dict, device="cuda:0"):
         if not torch.cuda.is_available():
