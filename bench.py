@@ -308,7 +308,7 @@ def main():
                    "algorithmic_bytes_per_launch": gemv_bytes(1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_M1_TRAFFIC_BYTES,
-                     "kernel": "gemv_i4g32_mfma_kernel<1,4,8,1,3,4096>", "wall_clock_us_per_step": round(wall1, 3)},
+                     "kernel": "gemv_i4g32_mfma_kernel<1,2,16,1,4,4096>", "wall_clock_us_per_step": round(wall1, 3)},
         "cpu_baseline": cpu,
         "parity": parity,
         "extras": extras,

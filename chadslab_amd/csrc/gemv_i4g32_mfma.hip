@@ -56,6 +56,7 @@ struct GemvCfg {
     static constexpr int SC_OFF = ZERO_OFF + ZERO_BYTES;
     static constexpr int SC_PPR = S * HP / 2;            // 16-byte pieces (8 groups) per scale tile row
     static constexpr int SC_PITCH = SC_PPR * 16 + 16;    // scale tile row: S*4*HP fp16 + pad
+    static constexpr int SC_NL = (P * SC_PPR + 63) / 64; // 16-byte scale loads per lane: the tile has 8*S pieces
     static constexpr int SC_WAVE = P * SC_PITCH;
     static constexpr int OPER_BYTES = SC_OFF + RBW * 4 * SC_WAVE;
     static constexpr int RED_BYTES = RBW * 4 * 64 * MP * 16;  // reuses the operand area after the K loop
@@ -107,8 +108,13 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
 
     // scale tile of this wave: P rows x 32*HP groups; lane -> (row, 8-group piece) for the single load
     uint8_t *sct = lds + C::SC_OFF + wave * C::SC_WAVE;
-    const int srow_l = lane / C::SC_PPR, spiece = lane % C::SC_PPR;  // lanes beyond P rows repeat the last row
-    const int srow = (n0 + srow_l < N) ? n0 + srow_l : N - 1;
+    int srow_l[C::SC_NL], spiece[C::SC_NL], srow[C::SC_NL];  // piece lane + 64*l; pieces beyond P rows repeat a valid row
+#pragma unroll
+    for (int l = 0; l < C::SC_NL; ++l) {
+        srow_l[l] = (lane + 64 * l) / C::SC_PPR;
+        spiece[l] = (lane + 64 * l) % C::SC_PPR;
+        srow[l] = (srow_l[l] < P && n0 + srow_l[l] < N) ? n0 + srow_l[l] : N - 1;
+    }
 
     // blockIdx.y selects a K range of kspan (a multiple of KC, or all of K) whose partial sums go to their own
     // [M,N] block of y: the split-K form for matrices with too few rows to fill the chip
@@ -137,9 +143,13 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
             }
 
         // 2. the wave's scale tile in one load.  Needs G % 8 == 0 (16-byte aligned pieces), checked on the host.
-        const int gs = (kc0 >> 5) + ks * S * 4 * HP + spiece * 8;
-        u32x4 sv = *reinterpret_cast<const u32x4 *>(sc + ((size_t)srow * G + (gs < G ? gs : 0)));
-        if (gs >= G) sv = u32x4{0, 0, 0, 0};
+        u32x4 sv[C::SC_NL];
+#pragma unroll
+        for (int l = 0; l < C::SC_NL; ++l) {
+            const int gs = (kc0 >> 5) + ks * S * 4 * HP + spiece[l] * 8;
+            sv[l] = *reinterpret_cast<const u32x4 *>(sc + ((size_t)srow[l] * G + (gs < G ? gs : 0)));
+            if (gs >= G) sv[l] = u32x4{0, 0, 0, 0};
+        }
 
         // 3. the wave's weight loads for the chunk: steps c = 8*ks + i, lane takes group (c*HP + h)*4 + j
         //    Only the first D are issued now; step i issues load i+D once its own data has arrived, so a
@@ -156,7 +166,9 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
         // 4. stage the activations: 16-byte pieces (8 k) -> [c][t][j][v], paired for the unpack order, and
         //    the C operands -136 * (sum of the group's 32 activations)
         __syncthreads();  // previous chunk's operand reads (or the zero fill) are done
-        if (srow_l < P) *reinterpret_cast<u32x4 *>(sct + srow_l * C::SC_PITCH + spiece * 16) = sv;  // wave-private tile
+#pragma unroll
+        for (int l = 0; l < C::SC_NL; ++l)  // wave-private tile
+            if (srow_l[l] < P) *reinterpret_cast<u32x4 *>(sct + srow_l[l] * C::SC_PITCH + spiece[l] * 16) = sv[l];
 #pragma unroll
         for (int p = 0; p < MP; ++p)
 #pragma unroll
@@ -293,19 +305,39 @@ int gemv_i4g32_mfma_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_
         float *ym = y + (size_t)m0 * N;
         int rc = 0;
         // <rows, K-parts, steps per wave, 4-wave groups per workgroup, prefetch distance>, picked by measurement
+        // Matrices with many rows run with 32 (M <= 4) or 64-row workgroups whose waves walk 16 steps of a chunk:
+        // half as many workgroups stage the activations and each wave's stream is twice as long.  Short matrices
+        // keep 16-row workgroups so that the grid still covers the chip.
+        const bool tall = N >= 8192;
         switch (mm) {
             case 1:
-                // rows of at most 2048 k: 2048-wide chunks, 4 steps per wave (no loads past the row)
-                rc = K <= 2048 ? launch_mfma<1, 4, 4, 1, 4, 2048>(xm, wp, sc, ym, N, K, st)
-                               : launch_mfma<1, 4, 8, 1, 3>(xm, wp, sc, ym, N, K, st);
+                if (K <= 2048)  // rows of at most 2048 k: 2048-wide chunks (no loads past the row)
+                    rc = tall ? launch_mfma<1, 2, 8, 1, 4, 2048>(xm, wp, sc, ym, N, K, st)
+                              : launch_mfma<1, 4, 4, 1, 4, 2048>(xm, wp, sc, ym, N, K, st);
+                else
+                    rc = tall ? launch_mfma<1, 2, 16, 1, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<1, 4, 8, 1, 3>(xm, wp, sc, ym, N, K, st);
                 break;
-            case 2: rc = launch_mfma<2, 2, 8, 1, 2>(xm, wp, sc, ym, N, K, st); break;
-            case 3: rc = launch_mfma<3, 1, 8, 1, 8>(xm, wp, sc, ym, N, K, st); break;
-            case 4: rc = launch_mfma<4, 1, 8, 1, 8>(xm, wp, sc, ym, N, K, st); break;
-            case 5: rc = launch_mfma<5, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st); break;
-            case 6: rc = launch_mfma<6, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st); break;
-            case 7: rc = launch_mfma<7, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st); break;
-            default: rc = launch_mfma<8, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st); break;
+            case 2:
+                rc = tall ? launch_mfma<2, 2, 16, 1, 3>(xm, wp, sc, ym, N, K, st) : launch_mfma<2, 2, 8, 1, 2>(xm, wp, sc, ym, N, K, st);
+                break;
+            case 3:
+                rc = tall ? launch_mfma<3, 1, 16, 1, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<3, 1, 8, 1, 8>(xm, wp, sc, ym, N, K, st);
+                break;
+            case 4:
+                rc = tall ? launch_mfma<4, 1, 16, 1, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<4, 1, 8, 1, 8>(xm, wp, sc, ym, N, K, st);
+                break;
+            case 5:
+                rc = tall ? launch_mfma<5, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<5, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
+                break;
+            case 6:
+                rc = tall ? launch_mfma<6, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<6, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
+                break;
+            case 7:
+                rc = tall ? launch_mfma<7, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<7, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
+                break;
+            default:
+                rc = tall ? launch_mfma<8, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<8, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
+                break;
         }
         if (rc != 0) return rc;
     }

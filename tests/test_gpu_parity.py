@@ -125,14 +125,22 @@ def test_gemv_int4_shapes(ops, m, n, k):
     assert O.rel_l2(y, O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_F32
 
 
-@pytest.mark.parametrize("m", [1, 4, 8])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8, 13])
 def test_gemv_int4_config1_full_size(ops, m):
     packed, s, xb, qw = i4_case(1001, m, 14336, 4096)
     y = ops.qgemv(bf16_tensor(xb), qw).cpu().numpy()
     assert O.rel_l2(y, O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_F32
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 14336, 4096), (8, 512, 4096), (4, 96, 256), (2, 40, 96)])
+@pytest.mark.parametrize("m,n,k", [(1, 32768, 2048), (1, 8200, 1024), (2, 8192, 8192), (5, 9001, 4096), (3, 8192, 256)])
+def test_gemv_int4_tall_matrices(ops, m, n, k):
+    # 8192 rows and more take the kernels with 32- and 64-row workgroups (a ragged last workgroup included)
+    packed, s, xb, qw = i4_case(3000 + n + k, m, n, k)
+    y = ops.qgemv(bf16_tensor(xb), qw).cpu().numpy()
+    assert np.isfinite(y).all() and O.rel_l2(y, O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_F32
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 14336, 4096), (2, 14336, 4096), (8, 512, 4096), (4, 96, 256), (2, 40, 96)])
 def test_gemv_int4_integer_accumulation_bit_exact(ops, m, n, k):
     from chadslab_amd import QWeightInt4G32
 
