@@ -43,6 +43,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=96)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the side measurements")
+    ap.add_argument("--extras", default="gemv,int8,gemm,moe,decode",
+                    help="comma list of the side measurements to run (gemv, int8, gemm, moe, decode)")
+    ap.add_argument("--short", action="store_true",
+                    help="few launches per side measurement: for hardware-counter runs, which serialise every dispatch")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run three 256 MiB device copies before the timed region: a kernel of known traffic "
                          "that hardware-counter runs scale FETCH_SIZE / WRITE_SIZE by")
@@ -125,14 +129,19 @@ def main():
     def gemv_bytes(m):
         return N * K // 2 + N * (K // 32) * 2 + m * K * 2 + m * N * 4
 
+    want = set() if args.no_extras else {e for e in args.extras.split(",") if e}
+    n_side = (48, 24) if args.short else (480, 48)   # launches, warm-up of the GEMV side measurements
+    n_gemm = (24, 24) if args.short else (240, 24)
+    n_moe = 3 if args.short else 20
+    n_dec = 4 if args.short else 64
     results = {}
     parity = {}
     for m in (1, 4, 8):
-        if m != 1 and args.no_extras:
+        if m != 1 and "gemv" not in want:
             continue
         x = torch.from_numpy(x_np[m]).to(torch.bfloat16).to(dev)
         y = torch.empty(m, N, dtype=torch.float32, device=dev)
-        steps = args.steps if m == 1 else min(args.steps, 480)
+        steps = args.steps if m == 1 else min(args.steps, n_side[0])
         us, wall = run_steps(lambda i: ops.qgemv(x, copies[i % N_COPIES], out=y), steps, args.warmup)
         results[m] = (us, wall, steps)
         if m == 1:
@@ -143,10 +152,10 @@ def main():
     achieved = gemv_bytes(1) / us1 * 1e-3  # GB/s
 
     extras = {}
-    if not args.no_extras:
+    if "gemv" in want:
         x1 = torch.from_numpy(x_np[1]).to(torch.bfloat16).to(dev)
         y1 = torch.empty(1, N, dtype=torch.float32, device=dev)
-        us_hot, _ = run_steps(lambda i: ops.qgemv(x1, base, out=y1), 480, 48)
+        us_hot, _ = run_steps(lambda i: ops.qgemv(x1, base, out=y1), *n_side)
         extras["gemv_i4g32"] = {
             "M%d" % m: {"us": round(results[m][0], 3), "GBps": round(gemv_bytes(m) / results[m][0] * 1e-3, 1),
                         "frac_hbm_peak": round(gemv_bytes(m) / results[m][0] * 1e-3 / HBM_PEAK_GBS, 4)}
@@ -157,7 +166,7 @@ def main():
             "note": "weights served by the 256 MB last-level cache, not HBM; not a roofline figure"}
     del copies
 
-    if not args.no_extras:
+    if "int8" in want:
         # config 0: int8 per-row GEMV
         N0, K0 = 16384, 2048
         r0 = np.random.Generator(np.random.PCG64(1000))
@@ -166,11 +175,12 @@ def main():
         s0 = torch.from_numpy(r0.uniform(0.001, 0.02, N0).astype(np.float32)).to(dev)
         c0 = [QWeightInt8(w0.clone(), s0.clone()) for _ in range(N_COPIES)]
         y0 = torch.empty(1, N0, dtype=torch.float32, device=dev)
-        us0, _ = run_steps(lambda i: ops.qgemv(x0, c0[i % N_COPIES], out=y0), 480, 48)
+        us0, _ = run_steps(lambda i: ops.qgemv(x0, c0[i % N_COPIES], out=y0), *n_side)
         b0 = N0 * K0 + N0 * 4 + K0 * 4 + N0 * 4
         extras["gemv_i8row_config0"] = {"us": round(us0, 3), "GBps": round(b0 / us0 * 1e-3, 1),
                                         "frac_hbm_peak": round(b0 / us0 * 1e-3 / HBM_PEAK_GBS, 4)}
         del c0, w0
+    if "gemm" in want:
         # config 2: prefill dequant-GEMM, int4 group-32 and int8 per-row
         M2, N2, K2 = 512, 4096, 4096
         r2 = np.random.Generator(np.random.PCG64(1002))
@@ -183,11 +193,12 @@ def main():
                          torch.from_numpy(r2.uniform(0.001, 0.02, N2).astype(np.float32)).to(dev))
         flop = 2.0 * M2 * N2 * K2
         for name, qw in (("gemm_i4g32_config2", q4), ("gemm_i8row_config2", q8)):
-            usg, _ = run_steps(lambda i: ops.qgemm(x2, qw, out=y2), 240, 24)
+            usg, _ = run_steps(lambda i: ops.qgemm(x2, qw, out=y2), *n_gemm)
             extras[name] = {"us": round(usg, 3), "TFLOPs": round(flop / usg * 1e-6, 1),
                             "frac_bf16_mfma_peak": round(flop / usg * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
         del x2, y2, q4, q8, p2, s2
+    if "moe" in want:
         # config 3: mixture-of-experts FFN, 8 experts, top-2, 256 tokens (weights random bytes: timing only, parity
         # is the test suite's job)
         T3, H3, F3, E3 = 256, 4096, 14336, 8
@@ -206,11 +217,11 @@ def main():
                 ops.moe_ffn(x3, z3, experts)
             a3, b3 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             a3.record(stream)
-            for _ in range(20):
+            for _ in range(n_moe):
                 ops.moe_ffn(x3, z3, experts)
             b3.record(stream)
             torch.cuda.synchronize()
-        us3 = a3.elapsed_time(b3) * 1000.0 / 20
+        us3 = a3.elapsed_time(b3) * 1000.0 / n_moe
         hit = int(torch.unique(ops.moe_route(z3, 2, True)[0]).numel())
         flop3 = 2.0 * T3 * 2 * 3 * H3 * F3
         bytes3 = hit * 3 * (F3 * H3 // 2 + F3 * (H3 // 32) * 2)
@@ -220,6 +231,7 @@ def main():
                                            "frac_hbm_peak": round(bytes3 / us3 * 1e-3 / HBM_PEAK_GBS, 4)}
         del experts, x3, z3
         torch.cuda.empty_cache()
+    if "decode" in want:
         # config 4: decode step, 18 layers, d 2048, 8 query heads x 256, 1 KV head, FFN 16384, vocab 256000, batch 1,
         # KV cache pre-filled to 2048 positions; 64 graph-replayed greedy steps (context 2048..2111)
         from chadslab_amd.decoder import DecoderConfig, QuantDecoder, random_weights
@@ -238,11 +250,11 @@ def main():
                 dec.graph.replay()
             a4, b4 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             a4.record(stream)
-            for _ in range(64):
+            for _ in range(n_dec):
                 dec.graph.replay()
             b4.record(stream)
             torch.cuda.synchronize()
-        us4 = a4.elapsed_time(b4) * 1000.0 / 64
+        us4 = a4.elapsed_time(b4) * 1000.0 / n_dec
         wbytes = sum(q.packed.numel() + 2 * q.scale.numel() for L in w4["layers"] for q in (L["wqkv"], L["wo"], L["wgu"], L["wd"]))
         wbytes += w4["emb"].packed.numel() + 2 * w4["emb"].scale.numel()
         kvbytes = cfg4.n_layers * 2 * 2080 * cfg4.dh * 2
