@@ -259,31 +259,44 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
         constexpr int set = decltype(set_c)::value;
         constexpr bool more1 = decltype(more1_c)::value, more2 = decltype(more2_c)::value;  // it+1 / it+2 exist
         const uint8_t *abase = ring + set * 4 * TL::SLOT_BYTES;
-#pragma unroll
-        for (int mb = 0; mb < 4; ++mb) {
-            // T(it, mb) has landed
-            if (more2) {
-                if (mb == 0) wait_vmcnt<3 * DPM + LPI>();
-                else wait_vmcnt<3 * DPM + LPI + NBL>();
-            } else if (more1) {
-                if (mb == 0) wait_vmcnt<3 * DPM + LPI>();
-                if (mb == 1) wait_vmcnt<2 * DPM + LPI>();
-                if (mb == 2) wait_vmcnt<1 * DPM + LPI>();
-                if (mb == 3) wait_vmcnt<LPI>();
-            } else {
-                if (mb == 0) wait_vmcnt<3 * DPM>();
-                if (mb == 1) wait_vmcnt<2 * DPM>();
-                if (mb == 2) wait_vmcnt<1 * DPM>();
-                if (mb == 3) wait_vmcnt<0>();
-            }
+        // The activation fragments of m-block mb+1 are read from LDS while the MFMAs of m-block mb run (a read
+        // placed right in front of its MFMA costs an exposed LDS round trip, 16 of them per iteration).
+        bf16x8 af[2][TL::T];
+        auto read_frags = [&](int buf, int mb) {
             const uint8_t *ab = abase + mb * TL::SLOT_BYTES;
 #pragma unroll
-            for (int t = 0; t < TL::T; ++t) {
-                const bf16x8 af = *reinterpret_cast<const bf16x8 *>(ab + nl * TL::ROWB + swz<TL>(nl, kq * TL::T + t) * 16);
+            for (int t = 0; t < TL::T; ++t)
+                af[buf][t] = *reinterpret_cast<const bf16x8 *>(ab + nl * TL::ROWB + swz<TL>(nl, kq * TL::T + t) * 16);
+        };
+        // T(it, 0) has landed: younger are the rest of its group, the group of it+1 (nothing issued yet by `it`)
+        if (more1) wait_vmcnt<3 * DPM + LPI>();
+        else wait_vmcnt<3 * DPM>();
+        read_frags(0, 0);
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) {
+            if (mb < 3) {
+                // T(it, mb+1) has landed.  Younger: T(it, mb+2..3), the group of it+1, and what `it` has issued so
+                // far: the refills of m-blocks 0..mb-1 and, once the first of them is out, the weights of it+2.
+                if (more2) {
+                    if (mb == 0) wait_vmcnt<2 * DPM + LPI>();
+                    else wait_vmcnt<2 * DPM + LPI + NBL>();
+                } else if (more1) {
+                    if (mb == 0) wait_vmcnt<2 * DPM + LPI>();
+                    if (mb == 1) wait_vmcnt<1 * DPM + LPI>();
+                    if (mb == 2) wait_vmcnt<LPI>();
+                } else {
+                    if (mb == 0) wait_vmcnt<2 * DPM>();
+                    if (mb == 1) wait_vmcnt<1 * DPM>();
+                    if (mb == 2) wait_vmcnt<0>();
+                }
+                read_frags((mb + 1) & 1, mb + 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < TL::T; ++t)
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb)
-                    acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bf[set][t][nb], acc[mb][nb], 0, 0, 0);
-            }
+                    acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mb & 1][t], bf[set][t][nb], acc[mb][nb], 0, 0, 0);
             if (more2) issue_dma(it + 2, mb);  // the slot just consumed
             // next iteration's weights become MFMA operands while this iteration's MFMAs run
             if (more1) {
