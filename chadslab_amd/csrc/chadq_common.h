@@ -1,5 +1,6 @@
 // Shared device helpers and the host-side error plumbing for libchadq (gfx950 only).
 #pragma once
+#include <atomic>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 

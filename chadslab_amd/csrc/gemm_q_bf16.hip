@@ -395,11 +395,11 @@ template <typename F, int NB, bool GUARD, bool OUTF32>
 static int launch_gemm_g(const uint16_t *x, const void *wq, const typename F::scale_t *sc, void *y, int M, int N,
                          int K, const GemmGroup *groups, int ngroups, hipStream_t st) {
     typedef Tile<F, NB> TL;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
+    if (!attr_set.load(std::memory_order_acquire)) {
         CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q_bf16_kernel<F, NB, GUARD, OUTF32>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, TL::LDS_BYTES));
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
     }
     const int tiles = ((N + TL::BN - 1) / TL::BN) * ((M + BM - 1) / BM);  // M = the largest group in a grouped launch
     const int grid = ((tiles + 7) / 8) * 8;  // a multiple of the 8 XCDs; surplus workgroups exit at once

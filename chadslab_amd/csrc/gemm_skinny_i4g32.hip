@@ -276,11 +276,11 @@ bool gemm_skinny_ok(int H, int F) { return H % 256 == 0 && F % 256 == 0; }
 template <int MODE>
 static int skinny_launch(const GemmGroup *groups, int E, int mtiles, int ntiles, int N, int K, int ksplit, size_t ystride,
                          hipStream_t st) {
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
+    if (!attr_set.load(std::memory_order_acquire)) {
         CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_skinny_i4g32_kernel<MODE>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS));
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL((gemm_skinny_i4g32_kernel<MODE>), dim3(ntiles, E * mtiles, ksplit), dim3(256), SK_LDS, st,
                        groups, E, N, K, K / ksplit, mtiles, ystride);

@@ -281,11 +281,11 @@ template <int MT, int HP, int S, int RBW, int D, int KC = 4096, bool XG = false>
 static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K,
                        hipStream_t st, int ksplit = 1) {
     typedef GemvCfg<MT, HP, S, RBW, KC> C;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
+    if (!attr_set.load(std::memory_order_acquire)) {
         CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XG>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::TOTAL));
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
     }
     const int units = (N + C::UR - 1) / C::UR;
     hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XG>), dim3((units + RBW - 1) / RBW, ksplit), dim3(256 * RBW),

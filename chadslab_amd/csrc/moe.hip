@@ -47,7 +47,13 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
     __shared__ int s_base[MOE_MAX_E];   // rows of expert e seen so far
     __shared__ int s_wave[16];          // per-wave counts of the current expert in the current chunk
     __shared__ int s_off[MOE_MAX_E + 1];
+    // expert and rank of every pair stay in LDS between the phases when they fit (a global write followed by a read
+    // from other threads costs a memory round trip per phase)
+    constexpr int LP = 4096;
+    __shared__ uint8_t s_e[LP];
+    __shared__ uint16_t s_r[LP];
     const int tid = threadIdx.x, B = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = B >> 6;
+    const bool in_lds = (T * top_k <= LP) && ws.pos;
     if (tid < MOE_MAX_E) s_base[tid] = 0;
 
     for (int t = tid; t < T; t += B) {
@@ -72,6 +78,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
         for (int j = 0; j < top_k; ++j) {
             idx[(size_t)t * top_k + j] = chosen[j];
             w[(size_t)t * top_k + j] = renorm ? pw[j] / wsum : pw[j];
+            if (in_lds) s_e[t * top_k + j] = (uint8_t)chosen[j];
         }
     }
     if (!ws.pos) return;  // routing only
@@ -80,7 +87,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
     const int P = T * top_k;
     for (int c0 = 0; c0 < P; c0 += B) {
         const int p = c0 + tid;
-        const int e_mine = p < P ? idx[p] : -1;
+        const int e_mine = p < P ? (in_lds ? (int)s_e[p] : idx[p]) : -1;
         int rank = 0;
         for (int e = 0; e < E; ++e) {
             const bool flag = (e_mine == e);
@@ -99,7 +106,10 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
             if (tid == 0) s_base[e] += total;
             __syncthreads();
         }
-        if (p < P) ws.pos[p] = rank;  // rank inside its expert for now
+        if (p < P) {  // rank inside its expert for now
+            if (in_lds) s_r[p] = (uint16_t)rank;
+            else ws.pos[p] = rank;
+        }
     }
     if (tid == 0) {
         int o = 0;
@@ -113,7 +123,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
     }
     __syncthreads();
     for (int p = tid; p < P; p += B) {
-        const int row = s_off[idx[p]] + ws.pos[p];
+        const int row = in_lds ? s_off[s_e[p]] + (int)s_r[p] : s_off[idx[p]] + ws.pos[p];
         ws.pos[p] = row;
         ws.tok[row] = p / top_k;
     }
@@ -222,7 +232,7 @@ int moe_ffn_i4g32_launch(const uint16_t *x, const float *logits, const chadq_moe
     }
     const int P = T * top_k;
     const int m_max = P < T ? P : T;  // an expert gets a token at most once
-    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 0, st, logits, ws.idx, ws.w, T, E, top_k, renorm, ws, ex, H, F);
+    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(T * top_k <= 1024 ? 256 : 1024), 0, st, logits, ws.idx, ws.w, T, E, top_k, renorm, ws, ex, H, F);
     hipLaunchKernelGGL(moe_gather_kernel, dim3(512), dim3(256), 0, st, x, ws.tok, ws.xs, P, H);
     int rc = hip_check(hipGetLastError(), "moe route/gather launch");
     if (rc) return rc;
