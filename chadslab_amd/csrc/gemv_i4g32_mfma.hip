@@ -66,12 +66,25 @@ struct GemvCfg {
 };
 
 // waves_per_eu(4): at most 128 VGPRs, which also makes the compiler pick the MFMA form that writes VGPRs.
-// XG: the activation vector is not given but formed while staging: x[k] = bf16( gelu_tanh(gu[k]) * gu[K + k] ) from
-// gu fp32 [2K] (`x` then points at gu) - the GeGLU of a gated FFN folded into its down projection.  M = 1 only.
-template <int MT, int HP, int S, int RBW, int D, int KC, bool XG = false>
+// XM: how the activation vector comes about (M = 1 for the modes other than 0).
+//   0  given: x bf16 [M,K].
+//   1  GeGLU folded in: x[k] = bf16( gelu_tanh(gu[k]) * gu[K + k] ) from gu fp32 [2K] (`x` points at gu) - a gated FFN's
+//      activation formed inside its down projection.
+//   2  residual add and RMSNorm folded in: r = pre.res + pre.delta[0] + .. + pre.delta[n-1] (fp32, in order),
+//      x = bf16( r / sqrt(mean(r^2) + eps) * pre.w ); the first workgroup also writes r to pre.res_out (a different
+//      buffer than pre.res: the other workgroups are still reading that one).  One chunk only (K <= KC).
+struct GemvPre {
+    const float *res, *delta, *w;
+    float *res_out;
+    int n;
+    float eps;
+};
+
+template <int MT, int HP, int S, int RBW, int D, int KC, int XM = 0>
 __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) void gemv_i4g32_mfma_kernel(
     const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
-    float *__restrict__ y, int N, int K, int kspan) {
+    float *__restrict__ y, int N, int K, int kspan, GemvPre pre) {
+    constexpr bool XG = (XM == 1), XN = (XM == 2);
     typedef GemvCfg<MT, HP, S, RBW, KC> C;
     constexpr int M = MT, MP = C::MP, MPASS = C::MPASS, P = C::P, KS = C::KS, T = C::T, XI = C::XI;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -124,6 +137,8 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
         // 1. activation loads FIRST.  Piece `it` = tid + T*q of pass p: row m = it / 512, i8 = it % 512.
         u32x4 xr[MP][XI];
         f32x4 gr[XG ? XI : 1][4];  // XG: 8 gate and 8 up values per piece
+        f32x4 nr[XN ? 12 : 1];     // XN: residual (2), norm weight (2), up to four delta vectors (8)
+        static_assert(!XN || (M == 1 && MP == 1 && KC / 8 == T), "the norm-folding mode stages one piece per thread");
 #pragma unroll
         for (int p = 0; p < MP; ++p)
 #pragma unroll
@@ -131,7 +146,19 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
                 const int m = (T * q) / (KC / 8);  // same for the whole workgroup: T divides KC/8
                 if (m >= MPASS || p * MPASS + m >= M) continue;  // compile time after unrolling
                 const int k = kc0 + 8 * ((tid + T * q) % (KC / 8));
-                if constexpr (XG) {
+                if constexpr (XN) {
+                    const int kk = k < K ? k : 0;
+                    nr[0] = *reinterpret_cast<const f32x4 *>(pre.res + kk);
+                    nr[1] = *reinterpret_cast<const f32x4 *>(pre.res + kk + 4);
+                    nr[2] = *reinterpret_cast<const f32x4 *>(pre.w + kk);
+                    nr[3] = *reinterpret_cast<const f32x4 *>(pre.w + kk + 4);
+#pragma unroll
+                    for (int jd = 0; jd < 4; ++jd) {  // absent vectors re-read the first one; they are not added
+                        const float *dp = (pre.n > 0 ? pre.delta : pre.res) + (size_t)(jd < pre.n ? jd : 0) * K + kk;
+                        nr[4 + 2 * jd] = *reinterpret_cast<const f32x4 *>(dp);
+                        nr[5 + 2 * jd] = *reinterpret_cast<const f32x4 *>(dp + 4);
+                    }
+                } else if constexpr (XG) {
                     const float *gp = reinterpret_cast<const float *>(x) + (k < K ? k : 0);
                     gr[q][0] = *reinterpret_cast<const f32x4 *>(gp);
                     gr[q][1] = *reinterpret_cast<const f32x4 *>(gp + 4);
@@ -165,6 +192,27 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
 
         // 4. stage the activations: 16-byte pieces (8 k) -> [c][t][j][v], paired for the unpack order, and
         //    the C operands -136 * (sum of the group's 32 activations)
+        float nv[8];
+        __shared__ float s_ss[4 * RBW];
+        if constexpr (XN) {
+            const int k = kc0 + 8 * (tid % (KC / 8));
+            float ss = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float v = nr[e >> 2][e & 3];
+#pragma unroll
+                for (int jd = 0; jd < 4; ++jd)
+                    if (jd < pre.n) v += nr[4 + 2 * jd + (e >> 2)][e & 3];
+                nv[e] = (k < K) ? v : 0.f;
+                ss += nv[e] * nv[e];
+            }
+            if (blockIdx.x == 0 && blockIdx.y == 0 && k < K) {
+                *reinterpret_cast<f32x4 *>(pre.res_out + k) = f32x4{nv[0], nv[1], nv[2], nv[3]};
+                *reinterpret_cast<f32x4 *>(pre.res_out + k + 4) = f32x4{nv[4], nv[5], nv[6], nv[7]};
+            }
+            ss = wave_sum_to_lane63(ss);
+            if (lane == 63) s_ss[wave] = ss;
+        }
         __syncthreads();  // previous chunk's operand reads (or the zero fill) are done
 #pragma unroll
         for (int l = 0; l < C::SC_NL; ++l)  // wave-private tile
@@ -177,7 +225,16 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
                 if (m >= MPASS || p * MPASS + m >= M) continue;  // padding row: its A lanes read the zero block
                 const int i8 = (tid + T * q) % (KC / 8);
                 u32x4 v;
-                if constexpr (XG) {
+                if constexpr (XN) {
+                    float tot = 0.f;
+#pragma unroll
+                    for (int wv2 = 0; wv2 < 4 * RBW; ++wv2) tot += s_ss[wv2];
+                    const float rinv = rsqrtf(tot / (float)K + pre.eps);
+                    uint32_t hb[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) hb[e] = f32_to_bf16_bits(nv[e] * rinv * nr[2 + (e >> 2)][e & 3]);
+                    v = u32x4{hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16), hb[4] | (hb[5] << 16), hb[6] | (hb[7] << 16)};
+                } else if constexpr (XG) {
                     const float g8[8] = {gr[q][0].x, gr[q][0].y, gr[q][0].z, gr[q][0].w, gr[q][1].x, gr[q][1].y, gr[q][1].z, gr[q][1].w};
                     const float u8[8] = {gr[q][2].x, gr[q][2].y, gr[q][2].z, gr[q][2].w, gr[q][3].x, gr[q][3].y, gr[q][3].z, gr[q][3].w};
                     uint32_t hb[8];
@@ -277,19 +334,19 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
 
 int gemv_i4g32_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
 
-template <int MT, int HP, int S, int RBW, int D, int KC = 4096, bool XG = false>
+template <int MT, int HP, int S, int RBW, int D, int KC = 4096, int XM = 0>
 static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K,
-                       hipStream_t st, int ksplit = 1) {
+                       hipStream_t st, int ksplit = 1, GemvPre pre = GemvPre{}) {
     typedef GemvCfg<MT, HP, S, RBW, KC> C;
     static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
     if (!attr_set.load(std::memory_order_acquire)) {
-        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XG>),
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::TOTAL));
         attr_set.store(true, std::memory_order_release);
     }
     const int units = (N + C::UR - 1) / C::UR;
-    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XG>), dim3((units + RBW - 1) / RBW, ksplit), dim3(256 * RBW),
-                       C::TOTAL, st, x, wp, sc, y, N, K, K / ksplit);
+    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM>), dim3((units + RBW - 1) / RBW, ksplit), dim3(256 * RBW),
+                       C::TOTAL, st, x, wp, sc, y, N, K, K / ksplit, pre);
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma launch");
 }
 
@@ -354,7 +411,16 @@ int gemv_i4g32_splitk_launch(const uint16_t *x, const uint8_t *wp, const uint16_
 // The same with x[k] = bf16( gelu_tanh(gu[k]) * gu[K + k] ) formed inside the kernel.
 int gemv_i4g32_splitk_geglu_launch(const float *gu, const uint8_t *wp, const uint16_t *sc, float *y_parts, int N, int K,
                                    int ksplit, hipStream_t st) {
-    return launch_mfma<1, 4, 8, 1, 3, 4096, true>(reinterpret_cast<const uint16_t *>(gu), wp, sc, y_parts, N, K, st, ksplit);
+    return launch_mfma<1, 4, 8, 1, 3, 4096, 1>(reinterpret_cast<const uint16_t *>(gu), wp, sc, y_parts, N, K, st, ksplit);
+}
+
+// y = W x with x = bf16(rmsnorm(res + sum of n delta vectors) * w) formed inside the kernel; res_out receives the sum.
+// K <= 2048 and a multiple of 256.
+int gemv_i4g32_addnorm_launch(const float *res, const float *delta, int n, const float *w, float eps, float *res_out,
+                              const uint8_t *wp, const uint16_t *sc, float *y, int N, int K, hipStream_t st) {
+    const GemvPre pre{res, delta, w, res_out, n, eps};
+    if (N >= 8192) return launch_mfma<1, 2, 8, 1, 4, 2048, 2>(nullptr, wp, sc, y, N, K, st, 1, pre);
+    return launch_mfma<1, 4, 4, 1, 4, 2048, 2>(nullptr, wp, sc, y, N, K, st, 1, pre);
 }
 
 }  // namespace chadq

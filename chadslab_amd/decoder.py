@@ -89,7 +89,8 @@ class QuantDecoder:
         f32, bf16, i32 = torch.float32, torch.bfloat16, torch.int32
         z = lambda n, dt: torch.zeros(n, dtype=dt, device=self.dev)  # noqa: E731
         c = cfg
-        self.x, self.xn = z(c.d, f32), z(c.d, bf16)
+        self.x, self.x2, self.xn = z(c.d, f32), z(c.d, f32), z(c.d, bf16)  # the residual stream ping-pongs between x and x2
+        self.fused_norm1 = c.d % 256 == 0 and c.d <= 2048  # first norm of a layer folded into the qkv projection
         self.qkv, self.q = z((c.hq + 2) * c.dh, f32), z(c.hq * c.dh, f32)
         self.att, self.ao = z(c.hq * c.dh, bf16), z(c.d, f32)
         # the down projection has few rows and a long K: split it over K when that fills the chip better
@@ -132,8 +133,16 @@ class QuantDecoder:
                                          self.x.data_ptr(), c.d, c.vocab, s), "chadq_embed_i4g32")
         pending = None
         for li, L in enumerate(self.w["layers"]):
-            self._norm(pending, L["ln1"])
-            self._gemv(self.xn, L["wqkv"], self.qkv)
+            if self.fused_norm1:
+                nd = 0 if pending is None else pending.numel() // c.d
+                _lib.check(lib.chadq_gemv_i4g32_addnorm(self.x.data_ptr(), pending.data_ptr() if nd else None, nd,
+                                                        L["ln1"].data_ptr(), c.eps, self.x2.data_ptr(),
+                                                        L["wqkv"].packed.data_ptr(), L["wqkv"].scale.data_ptr(),
+                                                        self.qkv.data_ptr(), L["wqkv"].N, c.d, s), "chadq_gemv_i4g32_addnorm")
+                self.x, self.x2 = self.x2, self.x  # the sum now lives in what was x2
+            else:
+                self._norm(pending, L["ln1"])
+                self._gemv(self.xn, L["wqkv"], self.qkv)
             if self.fused_attn:
                 _lib.check(lib.chadq_attn_decode_mqa_fused(self.qkv.data_ptr(), self.pos.data_ptr(), self.rope.data_ptr(),
                                                            self.kcache[li].data_ptr(), self.vcache[li].data_ptr(),
@@ -147,8 +156,15 @@ class QuantDecoder:
                                                      self.pos.data_ptr(), self.part.data_ptr(), self.att.data_ptr(), c.hq, c.dh,
                                                      c.max_ctx, s), "chadq_attn_decode_mqa")
             self._gemv(self.att, L["wo"], self.ao)
-            self._norm(self.ao, L["ln2"])
-            self._gemv(self.xn, L["wgu"], self.gu)
+            if self.fused_norm1:  # the second norm folds into the gate+up projection the same way
+                _lib.check(lib.chadq_gemv_i4g32_addnorm(self.x.data_ptr(), self.ao.data_ptr(), 1, L["ln2"].data_ptr(), c.eps,
+                                                        self.x2.data_ptr(), L["wgu"].packed.data_ptr(),
+                                                        L["wgu"].scale.data_ptr(), self.gu.data_ptr(), L["wgu"].N, c.d, s),
+                           "chadq_gemv_i4g32_addnorm")
+                self.x, self.x2 = self.x2, self.x
+            else:
+                self._norm(self.ao, L["ln2"])
+                self._gemv(self.xn, L["wgu"], self.gu)
             if self.ksplit > 1:  # GeGLU folded into the split-K down projection
                 _lib.check(lib.chadq_gemv_i4g32_splitk_geglu(self.gu.data_ptr(), L["wd"].packed.data_ptr(),
                                                              L["wd"].scale.data_ptr(), self.dn.data_ptr(), c.d, c.ffn,

@@ -97,6 +97,16 @@ int chadq_gemv_i4g32_splitk_geglu(const float *gu, const uint8_t *wp, const uint
                                   int ksplit, void *stream);
 
 /*
+ * chadq_add_rmsnorm_bf16 folded into the M = 1 product that consumes it: r = res + delta[0] + ... + delta[n_delta-1]
+ * (fp32, in order; delta fp32 [n_delta, K], n_delta <= 4), x = bf16( r / sqrt(mean(r^2) + eps) * norm_w ),
+ * y[n] = the int4 group-32 product of x with row n; r is written to res_out, which must be a different buffer
+ * than res (other workgroups still read res while the first one writes).  K a multiple of 256, K <= 2048;
+ * every array 16-byte aligned.
+ */
+int chadq_gemv_i4g32_addnorm(const float *res, const float *delta, int n_delta, const float *norm_w, float eps, float *res_out,
+                             const uint8_t *wp, const uint16_t *scale_f16, float *y, int N, int K, void *stream);
+
+/*
  * y[m,n] = scale[n] * sum_k x[m,k] * W[n,k]                                 (config 0)
  * x fp32 [M,K], W int8 [N,K], scale fp32 [N], y fp32 [M,N], 1 <= M <= 16, K % 16 == 0.
  */

@@ -102,6 +102,32 @@ def test_gemv_splitk_parts(lib, n, k, ksplit):
         chk(lib.chadq_gemv_i4g32_splitk(tx.data_ptr(), tp_.data_ptr(), ts.data_ptr(), parts.data_ptr(), n, k, 3, stream()), "splitk")
 
 
+@pytest.mark.parametrize("n,k,nd", [(2560, 2048, 4), (2560, 2048, 0), (100, 512, 1), (9000, 1024, 2), (32768, 2048, 1)])
+def test_gemv_addnorm_equals_norm_then_gemv(lib, n, k, nd):
+    r = rng(5 * n + k + nd)
+    u = r.integers(0, 16, (n, k), dtype=np.uint8)
+    packed = (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8)
+    s = r.lognormal(-5, 0.5, (n, k // 32)).astype(np.float16)
+    res = (r.standard_normal(k) * 2).astype(np.float32)
+    delta = r.standard_normal((max(nd, 1), k)).astype(np.float32)
+    w = (1 + 0.1 * r.standard_normal(k)).astype(np.float32)
+    tp_, ts, tr, td, tw = dev(packed), dev(s), dev(res), dev(delta), dev(w)
+    tro = torch.zeros(k, dtype=torch.float32, device=DEV)
+    y = torch.zeros(n, dtype=torch.float32, device=DEV)
+    chk(lib.chadq_gemv_i4g32_addnorm(tr.data_ptr(), td.data_ptr() if nd else None, nd, tw.data_ptr(), 1e-6, tro.data_ptr(),
+                                     tp_.data_ptr(), ts.data_ptr(), y.data_ptr(), n, k, stream()), "addnorm")
+    want_res = res.copy()
+    for j in range(nd):
+        want_res = want_res + delta[j]
+    assert np.array_equal(tro.cpu().numpy(), want_res)      # the residual sum, bit for bit
+    assert np.array_equal(tr.cpu().numpy(), res)            # the input residual is left alone
+    xb = O.f32_to_bf16(O.rmsnorm(want_res, w, 1e-6))[None, :]
+    assert O.rel_l2(y.cpu().numpy(), O.qgemm_int4g32_f64(xb, packed, s)[0]) < 3e-3  # bf16 ties may round the other way
+    with pytest.raises(ValueError):
+        chk(lib.chadq_gemv_i4g32_addnorm(tr.data_ptr(), None, 0, tw.data_ptr(), 1e-6, tr.data_ptr(), tp_.data_ptr(), ts.data_ptr(),
+                                         y.data_ptr(), n, k, stream()), "addnorm")
+
+
 @pytest.mark.parametrize("n,k,ksplit", [(2048, 16384, 4), (100, 8192, 1)])
 def test_gemv_splitk_geglu_equals_geglu_then_gemv(lib, n, k, ksplit):
     r = rng(3 * n + k + ksplit)
@@ -341,6 +367,13 @@ def test_decoder_step_small_graph_replay():
     from chadslab_amd.decoder import DecoderConfig
 
     _run_steps(DecoderConfig(n_layers=2, d=512, hq=4, dh=64, ffn=1024, vocab=1000, max_ctx=256), 41, 60, 5, True)
+
+
+def test_decoder_step_odd_layer_count_graph_replay():
+    from chadslab_amd.decoder import DecoderConfig
+
+    # three layers: the residual stream's two buffers end a step swapped; the captured graph must not care
+    _run_steps(DecoderConfig(n_layers=3, d=256, hq=2, dh=64, ffn=512, vocab=500, max_ctx=128), 44, 50, 4, True)
 
 
 def test_decoder_step_odd_sizes_generic_gemv():
