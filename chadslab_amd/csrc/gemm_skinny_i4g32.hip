@@ -54,11 +54,18 @@ struct SkDequant {
 // below count how many younger requests may still be outstanding.  Past the end of K the requests repeat the
 // first addresses so the counts stay uniform (their slots are never read).
 constexpr int SK_MB = SK_MT / 32;
+// Depth 2 keeps the rings at 76 KiB, two workgroups per CU.  Depth 4 (120 KiB, one workgroup per CU, twice the
+// bytes in flight per workgroup) measured 3 % slower on the benchmark's expert shapes: with one wave per SIMD the
+// LDS and barrier latencies of an iteration are no longer covered by a second workgroup.
+constexpr int SK_DA = 2;                // activation stages requested ahead (even)
+constexpr int SK_DB = SK_DA / 2;        // weight slots (two iterations each) requested ahead
+constexpr int SK_NSA = SK_DA + 1, SK_NSB = SK_DB + 1;
 constexpr int SK_ASTAGE = SK_MB * 32 * 128;
-constexpr int SK_A_BYTES = 3 * SK_ASTAGE;
+constexpr int SK_A_BYTES = SK_NSA * SK_ASTAGE;
 constexpr int SK_BSLOT = 64 * 64 + 64 * 16;
-constexpr int SK_B_WAVE = 2 * SK_BSLOT;
+constexpr int SK_B_WAVE = SK_NSB * SK_BSLOT;
 constexpr int SK_LDS = SK_A_BYTES + 4 * SK_B_WAVE;
+constexpr int SK_WGS_PER_CU = (2 * SK_LDS <= 160 * 1024) ? 2 : 1;
 
 template <int MODE, int MB>
 __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, const uint8_t *__restrict__ w0,
@@ -192,29 +199,43 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
         }
     };
 
-    // request order: A(0) B(0) A(1) | it=0: A(2) B(1) | it=1: A(3) | it=2: A(4) B(2) | ...
-    issue_a(0, 0);
-    issue_b(0, 0);
-    issue_a(1, 1);
-    int st = 0;  // it % 3
+    // Request groups: iteration e issues A(e + DA) and, when e is even, B(e/2 + DB) after it.  The prologue plays
+    // e = -DA .. -1.  Waiting for the group of iteration it - DA leaves the DA - 1 younger groups outstanding:
+    // they alternate odd (MB requests) and even (MB + 5), starting with the parity opposite to `it`.
+    constexpr int W_EVEN = (SK_DA / 2) * MB + (SK_DA / 2 - 1) * (MB + 5);  // younger: odd, even, ..., odd
+    constexpr int W_ODD = (SK_DA / 2) * (MB + 5) + (SK_DA / 2 - 1) * MB;   // younger: even, odd, ..., even
+    int sa_fill = 0, sb_fill = 0;  // next stage / slot to fill
+#pragma unroll
+    for (int e = -SK_DA; e < 0; ++e) {
+        issue_a(e + SK_DA, sa_fill);
+        sa_fill = sa_fill + 1 == SK_NSA ? 0 : sa_fill + 1;
+        if ((e & 1) == 0) {
+            issue_b(e / 2 + SK_DB, sb_fill);
+            sb_fill = sb_fill + 1 == SK_NSB ? 0 : sb_fill + 1;
+        }
+    }
+    int sa = 0, sb = 0;  // stage of iteration it, slot of iterations it, it+1
     for (int it = 0; it < nit; it += 2) {
-        const int m = it >> 1, st1 = st == 2 ? 0 : st + 1, st2 = st1 == 2 ? 0 : st1 + 1;
-        // even iteration: needs A(it) and B(m); only A(it+1) is younger
-        wait_vmcnt<MB>();
+        const int m = it >> 1;
+        wait_vmcnt<W_EVEN>();  // A(it) and B(m) have landed
         // the bare barrier instruction: __syncthreads() would add a fence that waits for every outstanding
         // request (vmcnt 0) and with it the whole prefetch
         __builtin_amdgcn_s_barrier();  // everybody's part of A(it) has landed; everybody is done reading A(it-1)
         __builtin_amdgcn_sched_barrier(0);
-        issue_a(it + 2, st2);          // into the stage of A(it-1)
-        issue_b(m + 1, (m + 1) & 1);   // into the slot of B(m-1), which this wave finished in iteration it-1
-        compute(st, m & 1, 0, kbeg + it * SK_KI);
-        // odd iteration: needs A(it+1); A(it+2) and B(m+1) are younger
-        wait_vmcnt<MB + 5>();
+        issue_a(it + SK_DA, sa_fill);  // into the stage of A(it-1)
+        sa_fill = sa_fill + 1 == SK_NSA ? 0 : sa_fill + 1;
+        issue_b(m + SK_DB, sb_fill);   // into the slot of B(m-1), which this wave finished in iteration it-1
+        sb_fill = sb_fill + 1 == SK_NSB ? 0 : sb_fill + 1;
+        compute(sa, sb, 0, kbeg + it * SK_KI);
+        sa = sa + 1 == SK_NSA ? 0 : sa + 1;
+        wait_vmcnt<W_ODD>();   // A(it+1) has landed
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        issue_a(it + 3, st);           // into the stage of A(it)
-        compute(st1, m & 1, 1, kbeg + (it + 1) * SK_KI);
-        st = st2;
+        issue_a(it + 1 + SK_DA, sa_fill);  // into the stage of A(it)
+        sa_fill = sa_fill + 1 == SK_NSA ? 0 : sa_fill + 1;
+        compute(sa, sb, 1, kbeg + (it + 1) * SK_KI);
+        sa = sa + 1 == SK_NSA ? 0 : sa + 1;
+        sb = sb + 1 == SK_NSB ? 0 : sb + 1;
     }
     wait_vmcnt<0>();  // the surplus requests of the last iterations must not outlive the workgroup's LDS
 
@@ -241,7 +262,7 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
 // groups: [E] gate, [E] up, [E] down descriptors as the router writes them.
 // grid: x = N tiles, y = expert * mtiles + token tile, z = K split (MODE 0 only).
 template <int MODE>
-__global__ __launch_bounds__(256, 2) void gemm_skinny_i4g32_kernel(const GemmGroup *__restrict__ groups, int E, int N, int K,
+__global__ __launch_bounds__(256, SK_WGS_PER_CU) void gemm_skinny_i4g32_kernel(const GemmGroup *__restrict__ groups, int E, int N, int K,
                                                                   int kspan, int mtiles, size_t ysplit_stride) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int g = blockIdx.y / mtiles, mt = blockIdx.y % mtiles;
