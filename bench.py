@@ -197,7 +197,15 @@ def main():
             extras[name] = {"us": round(usg, 3), "TFLOPs": round(flop / usg * 1e-6, 1),
                             "frac_bf16_mfma_peak": round(flop / usg * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
-        del x2, y2, q4, q8, p2, s2
+        # the kernel's asymptote at a larger M (not a benchmark config: extra, labelled as such)
+        M2b = 4096
+        x2b = torch.randn(M2b, K2, device=dev).to(torch.bfloat16)
+        y2b = torch.empty(M2b, N2, dtype=torch.bfloat16, device=dev)
+        usb, _ = run_steps(lambda i: ops.qgemm(x2b, q4, out=y2b), max(8, n_gemm[0] // 8), 4)
+        extras["gemm_i4g32_M4096_extra"] = {"us": round(usb, 2), "TFLOPs": round(2.0 * M2b * N2 * K2 / usb * 1e-6, 1),
+                                            "frac_bf16_mfma_peak": round(2.0 * M2b * N2 * K2 / usb * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                            "note": "same kernel at M=4096, N=K=4096: not a benchmark configuration"}
+        del x2, y2, q4, q8, p2, s2, x2b, y2b
     if "moe" in want:
         # config 3: mixture-of-experts FFN, 8 experts, top-2, 256 tokens (weights random bytes: timing only, parity
         # is the test suite's job)
