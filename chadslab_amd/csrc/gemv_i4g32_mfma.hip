@@ -83,7 +83,7 @@ struct GemvPre {
 template <int MT, int HP, int S, int RBW, int D, int KC, int XM = 0>
 __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) void gemv_i4g32_mfma_kernel(
     const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
-    float *__restrict__ y, int N, int K, int kspan, GemvPre pre) {
+    float *__restrict__ y, int N, int K, int kspan, int pv, GemvPre pre) {
     constexpr bool XG = (XM == 1), XN = (XM == 2);
     typedef GemvCfg<MT, HP, S, RBW, KC> C;
     constexpr int M = MT, MP = C::MP, MPASS = C::MPASS, P = C::P, KS = C::KS, T = C::T, XI = C::XI;
@@ -93,9 +93,11 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
     const int rbs = wv / KS, ks = wv % KS;         // row block inside the unit, K-slice
     const int nl = lane & 15, j = lane >> 4;
     const int h = nl / P, r = nl % P;              // K-part and row of this lane's MFMA column
-    const int n0 = (blockIdx.x * RBW + unit) * C::UR + rbs * P;
+    // A tile uses its first pv <= P rows (the host picks pv so that the workgroups fill whole rounds of the chip);
+    // the lanes of the other rows repeat the tile's first row and their sums are dropped.
+    const int n0 = ((blockIdx.x * RBW + unit) * (4 / KS) + rbs) * pv;
     const int KH = K >> 1, G = K >> 5;
-    const int row = (n0 + r < N) ? n0 + r : N - 1;
+    const int row = (r < pv && n0 + r < N) ? n0 + r : (n0 < N ? n0 : N - 1);
     const uint32_t wrow = (uint32_t)row * (uint32_t)KH;  // byte offset; the host checks N*K/2 < 2^31
     const uint32_t mask_r = vgpr_const(0x000F000Fu), magic_r = vgpr_const(kBf16Magic);
 
@@ -126,7 +128,7 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
     for (int l = 0; l < C::SC_NL; ++l) {
         srow_l[l] = (lane + 64 * l) / C::SC_PPR;
         spiece[l] = (lane + 64 * l) % C::SC_PPR;
-        srow[l] = (srow_l[l] < P && n0 + srow_l[l] < N) ? n0 + srow_l[l] : N - 1;
+        srow[l] = (srow_l[l] < pv && n0 + srow_l[l] < N) ? n0 + srow_l[l] : (n0 < N ? n0 : N - 1);
     }
 
     // blockIdx.y selects a K range of kspan (a multiple of KC, or all of K) whose partial sums go to their own
@@ -327,12 +329,42 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
                     const int wsrc = un * 4 + rb * KS + k4, lsrc = 16 * q + hh * P + rr;
                     t += reinterpret_cast<const float *>(red)[((wsrc * 64 + lsrc) * MP + p) * 4 + hh * MPASS + m];
                 }
-        const int nn = (blockIdx.x * RBW + un) * UR + n16, mm = p * MPASS + m;
-        if (nn < N && mm < M) y[(size_t)mm * N + nn] = t;
+        const int nn = ((blockIdx.x * RBW + un) * (4 / KS) + rb) * pv + rr, mm = p * MPASS + m;
+        if (rr < pv && nn < N && mm < M) y[(size_t)mm * N + nn] = t;
     }
 }
 
 int gemv_i4g32_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
+
+// Rows of a P-row tile to use.  All workgroups of these grids are resident at once, so the launch lasts as long as
+// the compute unit with the most workgroups: ceil(workgroups / CUs) of them.  Using a few rows less per tile can turn
+// 1.75 workgroups per CU (two on most, one on the rest) into exactly 2 shorter ones.  The fill is
+// N / (rounds * CUs * rows per workgroup); fewer rows are taken only for a gain of more than 5 %.
+static int pick_tile_rows(int N, int P, int tiles_per_wg, int ksplit) {
+    static std::atomic<int> n_cu{0};
+    int cus = n_cu.load(std::memory_order_relaxed);
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return P;
+        cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        n_cu.store(cus, std::memory_order_relaxed);
+    }
+    int best = P;
+    double fill_p = 0.0, best_fill = 0.0;
+    for (int pv = P; pv >= P - P / 4; --pv) {
+        const int64_t tiles = (N + pv - 1) / pv;
+        const int64_t wgs = (tiles + tiles_per_wg - 1) / tiles_per_wg * ksplit;
+        const int64_t rounds = (wgs + cus - 1) / cus;
+        const double fill = (double)N * ksplit / ((double)rounds * cus * pv * tiles_per_wg);
+        if (pv == P) fill_p = best_fill = fill;
+        if (fill > best_fill && fill > 1.05 * fill_p) {
+            best = pv;
+            best_fill = fill;
+        }
+    }
+    return best;
+}
 
 template <int MT, int HP, int S, int RBW, int D, int KC = 4096, int XM = 0>
 static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K,
@@ -344,9 +376,11 @@ static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::TOTAL));
         attr_set.store(true, std::memory_order_release);
     }
-    const int units = (N + C::UR - 1) / C::UR;
-    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM>), dim3((units + RBW - 1) / RBW, ksplit), dim3(256 * RBW),
-                       C::TOTAL, st, x, wp, sc, y, N, K, K / ksplit, pre);
+    const int tiles_per_wg = 4 / C::KS * RBW;
+    const int pv = pick_tile_rows(N, C::P, tiles_per_wg, ksplit);
+    const int tiles = (N + pv - 1) / pv;
+    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM>), dim3((tiles + tiles_per_wg - 1) / tiles_per_wg, ksplit),
+                       dim3(256 * RBW), C::TOTAL, st, x, wp, sc, y, N, K, K / ksplit, pv, pre);
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma launch");
 }
 

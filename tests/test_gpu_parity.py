@@ -132,9 +132,12 @@ def test_gemv_int4_config1_full_size(ops, m):
     assert O.rel_l2(y, O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_F32
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 32768, 2048), (1, 8200, 1024), (2, 8192, 8192), (5, 9001, 4096), (3, 8192, 256)])
+@pytest.mark.parametrize("m,n,k", [(1, 32768, 2048), (1, 8200, 1024), (2, 8192, 8192), (5, 9001, 4096), (3, 8192, 256),
+                                   (1, 11008, 4096), (2, 12345, 512), (4, 20000, 512), (8, 28672, 512), (1, 5000, 2048),
+                                   (7, 12345, 768)])
 def test_gemv_int4_tall_matrices(ops, m, n, k):
-    # 8192 rows and more take the kernels with 32- and 64-row workgroups (a ragged last workgroup included)
+    # 8192 rows and more take the kernels with 32- and 64-row workgroups (a ragged last workgroup included); row
+    # counts that would end mid-round on the chip run with tiles of 6, 7, 12, 13 or 14 rows instead of 8 or 16
     packed, s, xb, qw = i4_case(3000 + n + k, m, n, k)
     y = ops.qgemv(bf16_tensor(xb), qw).cpu().numpy()
     assert np.isfinite(y).all() and O.rel_l2(y, O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_F32
