@@ -70,6 +70,7 @@ int rope_table_launch(float *, int, int, float, hipStream_t);
 int attn_mqa_fused_launch(const float *, const int32_t *, const float *, uint16_t *, uint16_t *, float *, uint16_t *, int, int, int,
                           hipStream_t);
 int argmax_launch(const float *, int, float *, int32_t *, int32_t *, int32_t *, int, hipStream_t);
+int sample_topk_launch(const float *, int, int, float, const float *, float *, int32_t *, int32_t *, int32_t *, int, hipStream_t);
 
 }  // namespace chadq
 
@@ -331,6 +332,18 @@ int chadq_argmax_f32(const float *v, int n, void *scratch, int32_t *token, int32
     float *pv = reinterpret_cast<float *>(scratch);
     int32_t *pi = reinterpret_cast<int32_t *>(pv + 256);
     return argmax_launch(v, n, pv, pi, token, pos, advance, st);
+}
+
+int chadq_sample_topk_f32(const float *v, int n, int k, float temperature, const float *u, void *workspace, int32_t *token,
+                          int32_t *pos, int advance, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(n >= 1 && n <= 96 * 8192, CHADQ_ERR_SHAPE, "chadq_sample_topk_f32: n=%d (1..786432)", n);
+    CHADQ_REQUIRE(k >= 1 && k <= 64 && k <= n, CHADQ_ERR_SHAPE, "chadq_sample_topk_f32: k=%d (1..min(64, n))", k);
+    CHADQ_REQUIRE(temperature > 0.f && temperature < INFINITY, CHADQ_ERR_SHAPE, "chadq_sample_topk_f32: temperature %g", (double)temperature);
+    CHADQ_REQUIRE(v && u && workspace && token && (pos || !advance), CHADQ_ERR_NULL, "chadq_sample_topk_f32: null pointer");
+    float *cv = reinterpret_cast<float *>(workspace);
+    int32_t *ci = reinterpret_cast<int32_t *>(cv + 96 * 64);
+    return sample_topk_launch(v, n, k, temperature, u, cv, ci, token, pos, advance, st);
 }
 
 }  // extern "C"

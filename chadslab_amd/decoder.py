@@ -108,6 +108,10 @@ class QuantDecoder:
             self.part = z(self.lib.chadq_attn_decode_mqa_workspace_floats(c.hq, c.dh, c.max_ctx), f32)
         self.scratch = z(512, f32)
         self.token, self.pos = z(1, i32), z(1, i32)
+        # sampling: (top_k, temperature) or None for greedy; the uniform draw lives in device memory, refreshed per step
+        self.sampling = None
+        self.u, self.sample_ws = z(1, f32), z(49152 // 4, f32)
+        self.rng = torch.Generator(device=self.dev)
         self.kcache = [z(c.max_ctx * c.dh, bf16) for _ in range(c.n_layers)]
         self.vcache = [z(c.max_ctx * c.dh, bf16) for _ in range(c.n_layers)]
         self.graph = None
@@ -175,8 +179,24 @@ class QuantDecoder:
             pending = self.dn
         self._norm(pending, self.w["lnf"])
         self._gemv(self.xn, self.w["emb"], self.logits)
-        _lib.check(lib.chadq_argmax_f32(self.logits.data_ptr(), c.vocab, self.scratch.data_ptr(), self.token.data_ptr(),
-                                        self.pos.data_ptr(), 1, s), "chadq_argmax_f32")
+        if self.sampling is None:
+            _lib.check(lib.chadq_argmax_f32(self.logits.data_ptr(), c.vocab, self.scratch.data_ptr(), self.token.data_ptr(),
+                                            self.pos.data_ptr(), 1, s), "chadq_argmax_f32")
+        else:
+            k, temperature = self.sampling
+            _lib.check(lib.chadq_sample_topk_f32(self.logits.data_ptr(), c.vocab, k, temperature, self.u.data_ptr(),
+                                                 self.sample_ws.data_ptr(), self.token.data_ptr(), self.pos.data_ptr(), 1, s),
+                       "chadq_sample_topk_f32")
+
+    def set_sampling(self, top_k: int = 0, temperature: float = 1.0, seed: int = 0) -> None:
+        """top_k = 0: greedy (argmax).  Otherwise the next token is drawn from the top_k most likely ones at the given
+        temperature.  Call before capture(): a captured graph keeps the mode it was captured with."""
+        if self.graph is not None:
+            raise RuntimeError("set_sampling after capture(): the captured graph keeps its sampling mode")
+        if top_k < 0 or top_k > min(64, self.cfg.vocab) or not temperature > 0:
+            raise ValueError("top_k in 0..min(64, vocab) and temperature > 0 required")
+        self.sampling = (int(top_k), float(temperature)) if top_k > 0 else None
+        self.rng.manual_seed(seed)
 
     def capture(self) -> None:
         """Captures step() in a HIP graph (after one eager warm-up step whose effects are undone)."""
@@ -198,11 +218,14 @@ class QuantDecoder:
         self.graph = g
 
     def generate(self, first_token: int, pos: int, n: int) -> List[int]:
-        """Greedy decoding of n tokens starting from `first_token` at position `pos` (the cache holds pos rows)."""
+        """Decodes n tokens starting from `first_token` at position `pos` (the cache holds pos rows): greedy, or sampled
+        as set_sampling() says."""
         self.token.fill_(first_token)
         self.pos.fill_(pos)
         out = []
         for _ in range(n):
+            if self.sampling is not None:
+                self.u.uniform_(0.0, 1.0, generator=self.rng)  # eager, stream-ordered before the step or the replay
             if self.graph is not None:
                 self.graph.replay()
             else:

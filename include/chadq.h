@@ -214,6 +214,16 @@ int chadq_geglu_bf16(const float *gu, uint16_t *h_bf16, int F, void *stream);
  */
 int chadq_argmax_f32(const float *v, int n, void *scratch, int32_t *token, int32_t *pos, int advance, void *stream);
 
+/*
+ * Top-k sampling.  Candidates: the k largest of v[0..n), larger first, lower index first among equals (NaN is never
+ * a candidate).  p_j = exp((v_j - v_0) / temperature) in that order; token[0] = the first candidate whose running
+ * sum of p exceeds u[0] * (sum of p), u[0] in [0, 1) read from device memory at run time (so a captured graph draws
+ * afresh on every replay once the caller has rewritten it).  k = 1 is argmax.  pos[0] += 1 if advance != 0.
+ * 1 <= k <= min(64, n), n <= 786432, temperature > 0.  workspace: 49152 bytes.
+ */
+int chadq_sample_topk_f32(const float *v, int n, int k, float temperature, const float *u, void *workspace, int32_t *token,
+                          int32_t *pos, int advance, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -280,3 +280,20 @@ def decode_step(model, token, pos, kcache, vcache, hq, dh, eps=1e-6, base=10000.
         x = x + qgemv_int4g32(h, *L["wd"])[0]
     xn = f32_to_bf16(rmsnorm(x, model["lnf"], eps))[None, :]
     return qgemv_int4g32(xn, ep, es)[0]
+
+
+def sample_topk(v: np.ndarray, k: int, temperature: float, u: float) -> int:
+    """Top-k sampling as the product defines it: candidates are the k largest logits, larger first and lower index
+    first among equals (NaN never a candidate); p_j = exp((v_j - v_0) / temperature); the token is the first candidate
+    whose running sum of p exceeds u * sum(p).  float64 arithmetic."""
+    v = np.asarray(v, dtype=np.float64)
+    idx = np.arange(v.size)[~np.isnan(v)]
+    if idx.size == 0:
+        return 0
+    order = idx[np.lexsort((idx, -v[idx]))][:k]
+    top = v[order[0]]
+    if np.isneginf(top):
+        return int(order[0])
+    c = np.cumsum(np.exp((v[order] - top) / temperature))
+    hit = np.nonzero(c > u * c[-1])[0]
+    return int(order[hit[0]] if hit.size else order[-1])

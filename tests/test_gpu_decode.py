@@ -279,6 +279,49 @@ def test_argmax_and_advance(lib, n):
     assert int(tok.item()) == int(np.argmax(v)) and int(pos.item()) == 42
 
 
+def _sample_margin(v, k, temperature, u):
+    """Distance of u from the nearest interval boundary of the truncated softmax (float64), as a fraction of 1."""
+    idx = np.arange(v.size)[~np.isnan(v)]
+    order = idx[np.lexsort((idx, -v[idx].astype(np.float64)))][:k]
+    c = np.cumsum(np.exp((v[order].astype(np.float64) - float(v[order[0]])) / temperature))
+    return float(np.abs(c / c[-1] - u).min())
+
+
+@pytest.mark.parametrize("n,k,temperature", [(256000, 1, 1.0), (256000, 8, 0.7), (256000, 50, 1.0), (256000, 64, 1.3),
+                                             (1000, 64, 1.0), (97, 5, 0.5), (5, 5, 1.0), (1, 1, 1.0), (786432, 40, 1.0)])
+def test_sample_topk_matches_the_oracle(lib, n, k, temperature):
+    r = rng(1000 + n + k)
+    v = (r.standard_normal(n) * 3).astype(np.float32)
+    if n > 10:
+        v[[3, n - 2]] = v.max() + 0.5   # two equal best logits: index 3 comes first
+        v[5] = np.nan                   # never a candidate
+    t = dev(v)
+    ws = torch.zeros(49152 // 4, dtype=torch.float32, device=DEV)
+    tok = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    pos = torch.tensor([7], dtype=torch.int32, device=DEV)
+    checked = 0
+    for u in np.concatenate([[0.0, 0.999999], r.random(30)]).astype(np.float32):
+        ud = torch.tensor([u], dtype=torch.float32, device=DEV)
+        chk(lib.chadq_sample_topk_f32(t.data_ptr(), n, k, temperature, ud.data_ptr(), ws.data_ptr(), tok.data_ptr(),
+                                      pos.data_ptr(), 1, stream()), "sample_topk")
+        got = int(tok.item())
+        if _sample_margin(v, k, temperature, float(u)) > 1e-5:  # fp32 sums may land on the other side of a boundary
+            assert got == O.sample_topk(v, k, temperature, float(u)), (n, k, u)
+            checked += 1
+        assert 0 <= got < n
+    assert checked >= 25 and int(pos.item()) == 7 + 32
+
+
+def test_sample_topk_rejects_bad_arguments(lib):
+    t = dev(np.zeros(100, np.float32))
+    ws = torch.zeros(49152 // 4, dtype=torch.float32, device=DEV)
+    tok = torch.zeros(1, dtype=torch.int32, device=DEV)
+    u = torch.zeros(1, dtype=torch.float32, device=DEV)
+    for n, k, temp in [(100, 0, 1.0), (100, 65, 1.0), (10, 11, 1.0), (100, 5, 0.0), (786433, 5, 1.0)]:
+        assert lib.chadq_sample_topk_f32(t.data_ptr(), n, k, temp, u.data_ptr(), ws.data_ptr(), tok.data_ptr(), None, 0, stream()) != 0
+    assert lib.chadq_sample_topk_f32(t.data_ptr(), 100, 5, 1.0, None, ws.data_ptr(), tok.data_ptr(), None, 0, stream()) != 0
+
+
 def test_embed_row(lib):
     V, d = 50, 96
     p, s = O.quantize_int4_g32(rng(9).standard_normal((V, d)).astype(np.float32))
@@ -367,6 +410,26 @@ def test_decoder_step_small_graph_replay():
     from chadslab_amd.decoder import DecoderConfig
 
     _run_steps(DecoderConfig(n_layers=2, d=512, hq=4, dh=64, ffn=1024, vocab=1000, max_ctx=256), 41, 60, 5, True)
+
+
+def test_decoder_sampling_eager_and_graph_draw_the_same_tokens():
+    from chadslab_amd.decoder import DecoderConfig, QuantDecoder
+
+    cfg = DecoderConfig(n_layers=2, d=512, hq=4, dh=64, ffn=1024, vocab=1000, max_ctx=256)
+    m = _upload(_model(46, cfg))
+    runs = []
+    for use_graph, top_k in ((False, 20), (True, 20), (False, 0), (False, 1)):
+        dec = QuantDecoder(cfg, m, DEV)
+        dec.set_sampling(top_k=top_k, temperature=1.5, seed=1234)
+        if use_graph:
+            dec.capture()
+            with pytest.raises(RuntimeError):
+                dec.set_sampling(top_k=0)
+        runs.append(dec.generate(5, 0, 24))
+    sampled, replayed, greedy, top1 = runs
+    assert sampled == replayed  # same seed, same draws, whether the step is launched or replayed
+    assert top1 == greedy       # k = 1 is argmax
+    assert all(0 <= t < cfg.vocab for t in sampled) and sampled != greedy
 
 
 def test_decoder_step_odd_layer_count_graph_replay():

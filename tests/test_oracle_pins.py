@@ -412,3 +412,33 @@ def test_decode_step_against_independent_torch_model():
         assert O.rel_l2(lo, lt) < 2e-3  # both round through bf16 at the same places; fp32 summation orders differ
         assert int(lo.argmax()) == int(lt.argmax())
         tok = int(lo.argmax())
+
+
+def test_sample_topk_special_cases():
+    r = np.random.Generator(np.random.PCG64(77))
+    for _ in range(20):  # k = 1 is argmax with the lowest index among equals, whatever u and temperature are
+        v = r.integers(-3, 4, 50).astype(np.float32)
+        assert O.sample_topk(v, 1, 0.3, r.random()) == int(np.argmax(v))
+    v = np.array([1.0, 3.0, 3.0, 2.0], np.float32)  # equal logits: the lower index comes first and has the same weight
+    assert O.sample_topk(v, 2, 1.0, 0.0) == 1 and O.sample_topk(v, 2, 1.0, 0.49) == 1
+    assert O.sample_topk(v, 2, 1.0, 0.51) == 2 and O.sample_topk(v, 2, 1.0, 0.999) == 2
+    assert O.sample_topk(np.array([np.nan, 1.0, np.nan, 5.0]), 3, 1.0, 0.0) == 3  # NaN is never a candidate
+    assert O.sample_topk(np.array([np.nan, np.nan]), 2, 1.0, 0.5) == 0
+    assert O.sample_topk(np.array([-np.inf, -np.inf, -np.inf]), 2, 1.0, 0.9) == 0
+    assert O.sample_topk(np.array([0.0, 100.0, 0.0]), 3, 0.01, 0.999999) == 1  # a cold temperature is greedy
+
+
+def test_sample_topk_draws_the_truncated_softmax():
+    from scipy.special import softmax
+
+    r = np.random.Generator(np.random.PCG64(78))
+    v = r.standard_normal(12).astype(np.float32) * 2
+    k, temperature, draws = 5, 0.7, 20000
+    top = torch.topk(torch.from_numpy(v), k).indices.numpy()  # independent selection of the candidates
+    want = softmax(v[top].astype(np.float64) / temperature)
+    counts = np.zeros(12)
+    for j in range(draws):
+        counts[O.sample_topk(v, k, temperature, (j + 0.5) / draws)] += 1
+    assert counts.sum() == draws and set(np.nonzero(counts)[0]) <= set(top.tolist())
+    assert np.abs(counts[top] / draws - want).max() <= 1.5 / draws  # a uniform grid of u hits each interval to +-1
+
