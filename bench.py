@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16
 # HBM bytes per launch of the headline kernel from hardware counters (FETCH_SIZE, WRITE_SIZE, each scaled by what a
 # 256 MiB copy reads for it); the counter runs are summarised in profiles/gemv_i4g32_m1_config1_hbm_traffic.txt
-GEMV_M1_TRAFFIC_BYTES = 33234000
+GEMV_M1_TRAFFIC_BYTES = 33278000
 N_COPIES = 12
 SEG = 48                     # launches per captured graph
 
