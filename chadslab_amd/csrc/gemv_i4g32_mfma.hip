@@ -155,10 +155,15 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
                     nr[2] = *reinterpret_cast<const f32x4 *>(pre.w + kk);
                     nr[3] = *reinterpret_cast<const f32x4 *>(pre.w + kk + 4);
 #pragma unroll
-                    for (int jd = 0; jd < 4; ++jd) {  // absent vectors re-read the first one; they are not added
-                        const float *dp = (pre.n > 0 ? pre.delta : pre.res) + (size_t)(jd < pre.n ? jd : 0) * K + kk;
-                        nr[4 + 2 * jd] = *reinterpret_cast<const f32x4 *>(dp);
-                        nr[5 + 2 * jd] = *reinterpret_cast<const f32x4 *>(dp + 4);
+                    for (int jd = 0; jd < 4; ++jd) {  // pre.n is uniform: absent vectors cost no load
+                        if (jd < pre.n) {
+                            const float *dp = pre.delta + (size_t)jd * K + kk;
+                            nr[4 + 2 * jd] = *reinterpret_cast<const f32x4 *>(dp);
+                            nr[5 + 2 * jd] = *reinterpret_cast<const f32x4 *>(dp + 4);
+                        } else {
+                            nr[4 + 2 * jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+                            nr[5 + 2 * jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+                        }
                     }
                 } else if constexpr (XG) {
                     const float *gp = reinterpret_cast<const float *>(x) + (k < K ? k : 0);
