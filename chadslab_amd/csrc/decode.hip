@@ -6,6 +6,8 @@
 //   RMSNorm: y = x / sqrt(mean(x^2) + eps) * w.   RoPE: rotate-half, base 10000, on q and k.
 //   Attention: multi-query (1 KV head), scores / sqrt(head_dim), softmax in fp32, KV cache bf16.
 //   FFN: GeGLU with the tanh form of GELU.   Embedding: the tied int4 output table, dequantised row.
+#include <type_traits>
+
 #include "chadq_common.h"
 
 namespace chadq {
@@ -408,9 +410,10 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
 
     const bool live = c < lpr;
     const float scale = rsqrtf((float)dh);
+    // 32 partial dot products per lane (4 rows x 8 heads, index 8i + h) over the lane's 8 columns ...
+    float dots[32];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int pl = wave * 8 + 2 * i + hw;
         const uint32_t kk[4] = {kv[i].x, kv[i].y, kv[i].z, kv[i].w};
         float k8[8];
 #pragma unroll
@@ -419,12 +422,38 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
             k8[2 * e + 1] = live ? bf16_bits_to_f32(kk[e] >> 16) : 0.f;
         }
 #pragma unroll
-        for (int h = 0; h < 8; ++h) {
-            float acc = qa[h].x * k8[0] + qa[h].y * k8[1] + qa[h].z * k8[2] + qa[h].w * k8[3] + qb[h].x * k8[4] +
-                        qb[h].y * k8[5] + qb[h].z * k8[6] + qb[h].w * k8[7];
-            acc = half_wave_sum_hi(acc);
-            if (c == 16) s_sc[h][pl] = (p0 + pl < ctx && h < hq) ? acc * scale : -INFINITY;
+        for (int h = 0; h < 8; ++h)
+            dots[8 * i + h] = qa[h].x * k8[0] + qa[h].y * k8[1] + qa[h].z * k8[2] + qa[h].w * k8[3] + qb[h].x * k8[4] +
+                              qb[h].y * k8[5] + qb[h].z * k8[6] + qb[h].w * k8[7];
+    }
+    // ... summed over the 32 lanes of the half wave by halving: in the step with lane mask m a lane hands the half of
+    // its values whose index bit m differs from its own lane bit to lane ^ m and adds what it receives, so after
+    // five steps lane c holds the complete sum of index c: 31 exchanges instead of 32 five-step reductions.
+    // Masks 8, 2 and 1 are DPP moves (a rotation by 8 inside a 16-lane row is an exchange with lane ^ 8); 16 and 4 go
+    // through the LDS crossbar, all exchanges of a step issued before the first result is used.
+    auto halve = [&](auto m_c, auto n_c) {
+        constexpr int m = decltype(m_c)::value, n = decltype(n_c)::value;
+        const bool up = (c & m) != 0;
+        float got[n / 2];
+#pragma unroll
+        for (int j = 0; j < n / 2; ++j) {
+            const float send = up ? dots[j] : dots[j + n / 2];
+            if (m == 8) got[j] = dpp_f32<0x128, 0xF>(send);
+            else if (m == 2) got[j] = dpp_f32<0x4E, 0xF>(send);
+            else if (m == 1) got[j] = dpp_f32<0xB1, 0xF>(send);
+            else got[j] = __shfl_xor(send, m, 64);
         }
+#pragma unroll
+        for (int j = 0; j < n / 2; ++j) dots[j] = (up ? dots[j + n / 2] : dots[j]) + got[j];
+    };
+    halve(std::integral_constant<int, 16>{}, std::integral_constant<int, 32>{});
+    halve(std::integral_constant<int, 8>{}, std::integral_constant<int, 16>{});
+    halve(std::integral_constant<int, 4>{}, std::integral_constant<int, 8>{});
+    halve(std::integral_constant<int, 2>{}, std::integral_constant<int, 4>{});
+    halve(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{});
+    {
+        const int i = c >> 3, h = c & 7, pl = wave * 8 + 2 * i + hw;
+        s_sc[h][pl] = (p0 + pl < ctx && h < hq) ? dots[0] * scale : -INFINITY;
     }
     __syncthreads();
     {
