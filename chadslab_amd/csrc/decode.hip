@@ -143,7 +143,6 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(const float *__restrict__ 
 // Every global load of the workgroup (its K rows, its V columns, q) is issued before the first wait: the
 // kernel is one memory round trip plus a few hundred ALU operations per thread.
 constexpr int ATT_CS = 32;
-constexpr int ATT_MAX_NB = 2048;  // slices the combine kernel can hold weights for (context <= 65536)
 __global__ __launch_bounds__(256) void attn_mqa_partial_kernel(const float *__restrict__ q, const uint16_t *__restrict__ kc,
                                                                const uint16_t *__restrict__ vc, const int32_t *__restrict__ pos,
                                                                float *__restrict__ part, int hq, int dh, int max_ctx) {
@@ -238,43 +237,70 @@ __global__ __launch_bounds__(256) void attn_mqa_partial_kernel(const float *__re
     }
 }
 
+// Max over the 64 lanes of a wavefront, returned to every lane (DPP moves; a lane a move does not reach keeps its own).
+__device__ __forceinline__ float wave_max_all(float v) {
+#define CHADQ_MAX_STEP(CTRL, MASK) \
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, MASK, 0xF, false)));
+    CHADQ_MAX_STEP(0xB1, 0xF)   // quad_perm [1,0,3,2]
+    CHADQ_MAX_STEP(0x4E, 0xF)   // quad_perm [2,3,0,1]
+    CHADQ_MAX_STEP(0x141, 0xF)  // row_half_mirror
+    CHADQ_MAX_STEP(0x140, 0xF)  // row_mirror
+    CHADQ_MAX_STEP(0x142, 0xA)  // row_bcast15 into rows 1 and 3
+    CHADQ_MAX_STEP(0x143, 0xC)  // row_bcast31 into rows 2 and 3
+#undef CHADQ_MAX_STEP
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+__device__ __forceinline__ float lane_value(float v, int lane_index) {  // lane_index uniform
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane_index));
+}
+
 // out[h] = bf16( sum_b exp(m_b - M) * o_b / sum_b exp(m_b - M) * s_b ).  Workgroup (h, g): head h, columns
-// 64g..64g+63; its four waves take the slices b = w, w+4, ... so that all loads of a thread are independent and
-// in flight together, and meet in LDS.
+// 64g..64g+63; its four waves take the slices b = w, w+4, ...  Every wave works out M and the factors exp(m_b - M) for
+// itself, slice b in lane b % 64 (reductions on DPP moves, factors handed out with v_readlane), so the workgroup
+// meets only once, for the sum over the waves.  The loads of the first 64 slices do not depend on the position and
+// are issued together with it.
 __global__ __launch_bounds__(256) void attn_mqa_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ pos,
                                                                uint16_t *__restrict__ out, int hq, int dh, int max_ctx) {
-    const int ctx = min(max(pos[0], 0), max_ctx - 1) + 1, nb = (ctx + ATT_CS - 1) / ATT_CS, h = blockIdx.x, tid = threadIdx.x;
-    __shared__ float s_f[ATT_MAX_NB];
-    __shared__ float scratch[4];
+    const int nbmax = (max_ctx + ATT_CS - 1) / ATT_CS;  // slices the workspace holds
+    const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     __shared__ float s_num[4][64];
     const size_t stride = (size_t)hq * (dh + 2);
     const float *ph = part + (size_t)h * (dh + 2);
-    const int wave = tid >> 6, colw = blockIdx.y * 64 + (tid & 63), colc = colw < dh ? colw : dh - 1;
-    // the first 16 slices of this wave are requested before anything waits
+    const int colw = blockIdx.y * 64 + lane, colc = colw < dh ? colw : dh - 1;
     float pre[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int b = wave + 4 * i;
-        pre[i] = ph[(size_t)(b < nb ? b : 0) * stride + 2 + colc];
+        pre[i] = ph[(size_t)(b < nbmax ? b : nbmax - 1) * stride + 2 + colc];
     }
-    float m = -INFINITY;
-    for (int b = tid; b < nb; b += 256) m = fmaxf(m, ph[b * stride]);
-    const float M = block_max(m, scratch);
-    float den = 0.f;
-    for (int b = tid; b < nb; b += 256) {
-        const float f = __expf(ph[b * stride] - M);
-        s_f[b] = f;
-        den += f * ph[b * stride + 1];
-    }
-    den = block_sum(den, scratch);  // its barriers also publish s_f
+    const int bl = lane < nbmax ? lane : nbmax - 1;
+    const float m0 = ph[(size_t)bl * stride], l0 = ph[(size_t)bl * stride + 1];
+    const int ctx = min(max(pos[0], 0), max_ctx - 1) + 1, nb = (ctx + ATT_CS - 1) / ATT_CS;
+
+    float m = lane < nb ? m0 : -INFINITY;
+    for (int b = lane + 64; b < nb; b += 64) m = fmaxf(m, ph[(size_t)b * stride]);
+    const float M = wave_max_all(m);
+    const float f0 = lane < nb ? __expf(m0 - M) : 0.f;
+    float den = lane < nb ? f0 * l0 : 0.f;
     float num = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-        const int b = wave + 4 * i;
-        if (b < nb) num += s_f[b] * pre[i];
+        const int b = wave + 4 * i;  // < 64
+        if (b < nb) num += lane_value(f0, b) * pre[i];
     }
-    for (int b = wave + 64; b < nb; b += 4) num += s_f[b] * ph[(size_t)b * stride + 2 + colc];
-    s_num[wave][tid & 63] = num;
+    for (int base = 64; base < nb; base += 64) {  // contexts beyond 2048 positions
+        const int b = base + lane;
+        const bool in = b < nb;
+        const float mb = in ? ph[(size_t)b * stride] : -INFINITY, lb = in ? ph[(size_t)b * stride + 1] : 0.f;
+        const float f = in ? __expf(mb - M) : 0.f;
+        den += f * lb;
+        for (int j = wave; j < 64 && base + j < nb; j += 4) num += lane_value(f, j) * ph[(size_t)(base + j) * stride + 2 + colc];
+    }
+    den = wave_sum_to_lane63(den);
+    den = lane_value(den, 63);
+    s_num[wave][lane] = num;
     __syncthreads();
     if (tid < 64 && colw < dh) {
         const float t = s_num[0][tid] + s_num[1][tid] + s_num[2][tid] + s_num[3][tid];
@@ -308,8 +334,10 @@ __device__ __forceinline__ float half_wave_sum_hi(float v) {
 }
 
 // Workgroup b: positions [32b, 32b+32).  qkv fp32 = [hq*dh | dh | dh] straight from the projection.  Every
-// workgroup rotates q itself (table lookup); the one that owns position pos also rotates k, writes row pos of both
-// caches and uses the new row from registers/LDS instead of reading it back.  Partials as attn_mqa_partial_kernel;
+// workgroup rotates q itself (table lookup): thread (head, 8-column piece) rotates its piece once and the rotated q
+// goes through LDS, so a thread issues 8 loads for q instead of 36; the V slice is fetched with 16-byte loads and
+// read by columns from LDS.  The workgroup that owns position pos also rotates k, writes row pos of both caches and
+// puts the new rows into LDS instead of reading them back.  Partials as attn_mqa_partial_kernel;
 // attn_mqa_combine_kernel follows.  (Letting the last workgroup to finish do the combination in the same launch
 // was tried and lost: one workgroup pulling every partial through one CU took longer than a second launch.)
 __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__restrict__ qkv, const int32_t *__restrict__ pos,
@@ -321,18 +349,20 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
     if (p0 >= ctx) return;
     const bool own = (p - p0) < ATT_CS;  // this slice contains the new position
     float *part = ws;
-    __shared__ __attribute__((aligned(16))) float s_sc[8][ATT_CS];  // scores, then probabilities
-    __shared__ __attribute__((aligned(16))) uint16_t s_krow[256];
+    __shared__ __attribute__((aligned(16))) float s_sc[8][ATT_CS];       // scores, then probabilities
+    __shared__ __attribute__((aligned(16))) float s_q[8][256];           // rotated q
+    __shared__ __attribute__((aligned(16))) uint16_t s_v[ATT_CS][256];   // the slice of V
+    __shared__ __attribute__((aligned(16))) uint16_t s_krow[256];        // the new (rotated) k row
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int half = dh >> 1, hw = lane >> 5, c = lane & 31, lpr = dh >> 3;
 
-    // V: thread t owns column t of every row of the slice
-    const int col = tid < dh ? tid : dh - 1;
-    uint16_t vv[ATT_CS];
+    // V: 16-byte pieces of the slice, piece ch = row * lpr + column piece, dealt round robin to the threads
+    u32x4 vld[4];
 #pragma unroll
-    for (int i = 0; i < ATT_CS; ++i) {
-        const int pi = (p0 + i < ctx) ? p0 + i : ctx - 1;
-        vv[i] = vc[(size_t)pi * dh + col];
+    for (int j = 0; j < 4; ++j) {
+        const int ch = tid + 256 * j, row = ch / lpr, vcc = ch % lpr;
+        const int pi = (p0 + row < ctx) ? p0 + row : ctx - 1;
+        if (row < ATT_CS) vld[j] = *reinterpret_cast<const u32x4 *>(vc + (size_t)pi * dh + vcc * 8);
     }
     // K: wave w owns rows 8w..8w+7 of the slice, two rows per load instruction
     const int cc = c < lpr ? c : 0;
@@ -343,22 +373,18 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
         const int pi = (p0 + pl < ctx) ? p0 + pl : ctx - 1;
         kv[i] = *reinterpret_cast<const u32x4 *>(kc + (size_t)pi * dh + cc * 8);
     }
-    // q: the lane's 8 columns of every head, the 8 columns they rotate with, and the angles
-    const int colq = cc * 8, lo = colq < half;
+    // q: thread (head tid/32, piece tid%32) loads its 8 columns, the 8 columns they rotate with, and the angles
+    const int qh = tid >> 5, qc = (tid & 31) < lpr ? (tid & 31) : 0;
+    const bool qlive = qh < hq && (tid & 31) < lpr;
+    const int colq = qc * 8, lo = colq < half;
     const int colp = lo ? colq + half : colq - half;  // partner columns
     const int jt = lo ? colq : colq - half;           // rotation index of element 0
-    f32x4 qa[8], qb[8], pa[8], pb[8];
-#pragma unroll
-    for (int h = 0; h < 8; ++h) {
-        const float *qh = qkv + (size_t)(h < hq ? h : 0) * dh;
-        qa[h] = *reinterpret_cast<const f32x4 *>(qh + colq);
-        qb[h] = *reinterpret_cast<const f32x4 *>(qh + colq + 4);
-        pa[h] = *reinterpret_cast<const f32x4 *>(qh + colp);
-        pb[h] = *reinterpret_cast<const f32x4 *>(qh + colp + 4);
-    }
+    const float *qrow = qkv + (size_t)(qh < hq ? qh : 0) * dh;
+    const f32x4 qa = *reinterpret_cast<const f32x4 *>(qrow + colq), qb = *reinterpret_cast<const f32x4 *>(qrow + colq + 4);
+    const f32x4 pa = *reinterpret_cast<const f32x4 *>(qrow + colp), pb = *reinterpret_cast<const f32x4 *>(qrow + colp + 4);
     const float *tp = table + ((size_t)p * half + jt) * 2;
-    f32x4 t0 = *reinterpret_cast<const f32x4 *>(tp), t1 = *reinterpret_cast<const f32x4 *>(tp + 4),
-          t2 = *reinterpret_cast<const f32x4 *>(tp + 8), t3 = *reinterpret_cast<const f32x4 *>(tp + 12);
+    const f32x4 t0 = *reinterpret_cast<const f32x4 *>(tp), t1 = *reinterpret_cast<const f32x4 *>(tp + 4),
+                t2 = *reinterpret_cast<const f32x4 *>(tp + 8), t3 = *reinterpret_cast<const f32x4 *>(tp + 12);
     // the owner's new K/V row
     float ka = 0.f, kb = 0.f, kcs = 1.f, ksn = 0.f, vnew = 0.f;
     if (own) {
@@ -372,6 +398,27 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
     }
     __builtin_amdgcn_sched_barrier(0);
 
+    // rotate q: low columns a*cos - b*sin, high columns b*cos + a*sin, (a, b) = (low, high) element of the pair
+    {
+        const float cs[8] = {t0.x, t0.z, t1.x, t1.z, t2.x, t2.z, t3.x, t3.z};
+        const float sn[8] = {t0.y, t0.w, t1.y, t1.w, t2.y, t2.w, t3.y, t3.w};
+        const float sg = lo ? -1.f : 1.f;
+        const float own8[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+        const float par8[8] = {pa.x, pa.y, pa.z, pa.w, pb.x, pb.y, pb.z, pb.w};
+        float r[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r[e] = qlive ? own8[e] * cs[e] + sg * par8[e] * sn[e] : 0.f;
+        if ((tid & 31) < lpr) {  // heads past hq hold zeros
+            *reinterpret_cast<f32x4 *>(&s_q[qh][colq]) = f32x4{r[0], r[1], r[2], r[3]};
+            *reinterpret_cast<f32x4 *>(&s_q[qh][colq + 4]) = f32x4{r[4], r[5], r[6], r[7]};
+        }
+    }
+    // the V slice into LDS; the owner's new row replaces the (not yet written) cache row
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int ch = tid + 256 * j, row = ch / lpr, vcc = ch % lpr;
+        if (row < ATT_CS && !(own && p0 + row == p)) *reinterpret_cast<u32x4 *>(&s_v[row][vcc * 8]) = vld[j];
+    }
     if (own) {
         if (tid < half) {
             const uint16_t ra = (uint16_t)f32_to_bf16_bits(ka * kcs - kb * ksn), rb = (uint16_t)f32_to_bf16_bits(kb * kcs + ka * ksn);
@@ -380,51 +427,44 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
             kc[(size_t)p * dh + tid] = ra;
             kc[(size_t)p * dh + tid + half] = rb;
         }
-        const uint16_t vb16 = (uint16_t)f32_to_bf16_bits(vnew);
-        if (tid < dh) vc[(size_t)p * dh + tid] = vb16;
-#pragma unroll
-        for (int i = 0; i < ATT_CS; ++i)
-            if (p0 + i == p) vv[i] = vb16;
-        __syncthreads();
+        if (tid < dh) {
+            const uint16_t vb16 = (uint16_t)f32_to_bf16_bits(vnew);
+            vc[(size_t)p * dh + tid] = vb16;
+            s_v[p - p0][tid] = vb16;
+        }
+    }
+    __syncthreads();
+    if (own) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             if (p0 + wave * 8 + 2 * i + hw == p) kv[i] = *reinterpret_cast<const u32x4 *>(s_krow + cc * 8);
-    }
-
-    // rotate q: low columns a*cos - b*sin, high columns b*cos + a*sin, (a, b) = (low, high) element of the pair
-    {
-        const float cs[8] = {t0.x, t0.z, t1.x, t1.z, t2.x, t2.z, t3.x, t3.z};
-        const float sn[8] = {t0.y, t0.w, t1.y, t1.w, t2.y, t2.w, t3.y, t3.w};
-        const float sg = lo ? -1.f : 1.f;
-#pragma unroll
-        for (int h = 0; h < 8; ++h) {
-            const float own8[8] = {qa[h].x, qa[h].y, qa[h].z, qa[h].w, qb[h].x, qb[h].y, qb[h].z, qb[h].w};
-            const float par8[8] = {pa[h].x, pa[h].y, pa[h].z, pa[h].w, pb[h].x, pb[h].y, pb[h].z, pb[h].w};
-            float r[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) r[e] = own8[e] * cs[e] + sg * par8[e] * sn[e];
-            qa[h] = f32x4{r[0], r[1], r[2], r[3]};
-            qb[h] = f32x4{r[4], r[5], r[6], r[7]};
-        }
     }
 
     const bool live = c < lpr;
     const float scale = rsqrtf((float)dh);
     // 32 partial dot products per lane (4 rows x 8 heads, index 8i + h) over the lane's 8 columns ...
     float dots[32];
+    {
+        f32x4 qra[8], qrb[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t kk[4] = {kv[i].x, kv[i].y, kv[i].z, kv[i].w};
-        float k8[8];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            k8[2 * e] = live ? bf16_bits_to_f32(kk[e] & 0xFFFFu) : 0.f;
-            k8[2 * e + 1] = live ? bf16_bits_to_f32(kk[e] >> 16) : 0.f;
+        for (int h = 0; h < 8; ++h) {
+            qra[h] = *reinterpret_cast<const f32x4 *>(&s_q[h][cc * 8]);
+            qrb[h] = *reinterpret_cast<const f32x4 *>(&s_q[h][cc * 8 + 4]);
         }
 #pragma unroll
-        for (int h = 0; h < 8; ++h)
-            dots[8 * i + h] = qa[h].x * k8[0] + qa[h].y * k8[1] + qa[h].z * k8[2] + qa[h].w * k8[3] + qb[h].x * k8[4] +
-                              qb[h].y * k8[5] + qb[h].z * k8[6] + qb[h].w * k8[7];
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t kk[4] = {kv[i].x, kv[i].y, kv[i].z, kv[i].w};
+            float k8[8];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                k8[2 * e] = live ? bf16_bits_to_f32(kk[e] & 0xFFFFu) : 0.f;
+                k8[2 * e + 1] = live ? bf16_bits_to_f32(kk[e] >> 16) : 0.f;
+            }
+#pragma unroll
+            for (int h = 0; h < 8; ++h)
+                dots[8 * i + h] = qra[h].x * k8[0] + qra[h].y * k8[1] + qra[h].z * k8[2] + qra[h].w * k8[3] + qrb[h].x * k8[4] +
+                                  qrb[h].y * k8[5] + qrb[h].z * k8[6] + qrb[h].w * k8[7];
+        }
     }
     // ... summed over the 32 lanes of the half wave by halving: in the step with lane mask m a lane hands the half of
     // its values whose index bit m differs from its own lane bit to lane ^ m and adds what it receives, so after
@@ -460,11 +500,20 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
         // softmax of the slice: thread -> (head tid/32, position tid%32)
         const int h = tid >> 5, i = tid & 31;
         const float s = s_sc[h][i];
+        // over the 32 positions: rotations inside the 16-lane rows (DPP), then one exchange between the two rows
         float mx = s;
-        for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        mx = fmaxf(mx, dpp_f32<0x128, 0xF>(mx));  // row_ror:8
+        mx = fmaxf(mx, dpp_f32<0x124, 0xF>(mx));  // row_ror:4
+        mx = fmaxf(mx, dpp_f32<0x122, 0xF>(mx));  // row_ror:2
+        mx = fmaxf(mx, dpp_f32<0x121, 0xF>(mx));  // row_ror:1
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         const float pr = (h < hq) ? __expf(s - mx) : 0.f;
         float sum = pr;
-        for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+        sum += dpp_f32<0x128, 0xF>(sum);
+        sum += dpp_f32<0x124, 0xF>(sum);
+        sum += dpp_f32<0x122, 0xF>(sum);
+        sum += dpp_f32<0x121, 0xF>(sum);
+        sum += __shfl_xor(sum, 16, 64);
         s_sc[h][i] = pr;
         if (i == 0 && h < hq) {
             float *dst = part + ((size_t)blockIdx.x * hq + h) * (dh + 2);
@@ -473,11 +522,13 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
         }
     }
     __syncthreads();
+    // V: thread t owns column t of every row of the slice
+    const int col = tid < dh ? tid : dh - 1;
     float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < ATT_CS; i += 4) {
-        const float v0 = bf16_bits_to_f32(vv[i]), v1 = bf16_bits_to_f32(vv[i + 1]), v2 = bf16_bits_to_f32(vv[i + 2]),
-                    v3 = bf16_bits_to_f32(vv[i + 3]);
+        const float v0 = bf16_bits_to_f32(s_v[i][col]), v1 = bf16_bits_to_f32(s_v[i + 1][col]),
+                    v2 = bf16_bits_to_f32(s_v[i + 2][col]), v3 = bf16_bits_to_f32(s_v[i + 3][col]);
 #pragma unroll
         for (int h = 0; h < 8; ++h) {
             const f32x4 p4 = *reinterpret_cast<const f32x4 *>(&s_sc[h][i]);
@@ -489,7 +540,6 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
         for (int h = 0; h < 8; ++h)
             if (h < hq) part[((size_t)blockIdx.x * hq + h) * (dh + 2) + 2 + tid] = o[h];
     }
-
 }
 
 // h = bf16( gelu_tanh(g) * u ), gu = [g(F) | u(F)] fp32
