@@ -140,7 +140,8 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
         u32x4 xr[MP][XI];
         f32x4 gr[XG ? XI : 1][4];  // XG: 8 gate and 8 up values per piece
         f32x4 nr[XN ? 12 : 1];     // XN: residual (2), norm weight (2), up to four delta vectors (8)
-        static_assert(!XN || (M == 1 && MP == 1 && KC / 8 == T), "the norm-folding mode stages one piece per thread");
+        static_assert(!XN || (M == 1 && MP == 1 && KC / 8 <= T), "the norm-folding mode stages one piece per thread");
+        const bool stager = !XN || tid < KC / 8;  // XN in a workgroup of more than KC/8 threads: the first KC/8 stage
 #pragma unroll
         for (int p = 0; p < MP; ++p)
 #pragma unroll
@@ -149,6 +150,7 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
                 if (m >= MPASS || p * MPASS + m >= M) continue;  // compile time after unrolling
                 const int k = kc0 + 8 * ((tid + T * q) % (KC / 8));
                 if constexpr (XN) {
+                    if (!stager) continue;  // whole waves
                     const int kk = k < K ? k : 0;
                     nr[0] = *reinterpret_cast<const f32x4 *>(pre.res + kk);
                     nr[1] = *reinterpret_cast<const f32x4 *>(pre.res + kk + 4);
@@ -210,10 +212,10 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
 #pragma unroll
                 for (int jd = 0; jd < 4; ++jd)
                     if (jd < pre.n) v += nr[4 + 2 * jd + (e >> 2)][e & 3];
-                nv[e] = (k < K) ? v : 0.f;
+                nv[e] = (k < K && stager) ? v : 0.f;
                 ss += nv[e] * nv[e];
             }
-            if (blockIdx.x == 0 && blockIdx.y == 0 && k < K) {
+            if (blockIdx.x == 0 && blockIdx.y == 0 && k < K && stager) {
                 *reinterpret_cast<f32x4 *>(pre.res_out + k) = f32x4{nv[0], nv[1], nv[2], nv[3]};
                 *reinterpret_cast<f32x4 *>(pre.res_out + k + 4) = f32x4{nv[4], nv[5], nv[6], nv[7]};
             }
@@ -230,6 +232,7 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
             for (int q = 0; q < XI; ++q) {
                 const int m = (T * q) / (KC / 8);
                 if (m >= MPASS || p * MPASS + m >= M) continue;  // padding row: its A lanes read the zero block
+                if (XN && !stager) continue;                     // whole waves
                 const int i8 = (tid + T * q) % (KC / 8);
                 u32x4 v;
                 if constexpr (XN) {
@@ -450,7 +453,8 @@ int gemv_i4g32_splitk_launch(const uint16_t *x, const uint8_t *wp, const uint16_
 // The same with x[k] = bf16( gelu_tanh(gu[k]) * gu[K + k] ) formed inside the kernel.
 int gemv_i4g32_splitk_geglu_launch(const float *gu, const uint8_t *wp, const uint16_t *sc, float *y_parts, int N, int K,
                                    int ksplit, hipStream_t st) {
-    return launch_mfma<1, 4, 8, 1, 3, 4096, 1>(reinterpret_cast<const uint16_t *>(gu), wp, sc, y_parts, N, K, st, ksplit);
+    // 8-wave workgroups: a compute unit forms its K range of the gated activation once instead of twice
+    return launch_mfma<1, 4, 8, 2, 3, 4096, 1>(reinterpret_cast<const uint16_t *>(gu), wp, sc, y_parts, N, K, st, ksplit);
 }
 
 // y = W x with x = bf16(rmsnorm(res + sum of n delta vectors) * w) formed inside the kernel; res_out receives the sum.
@@ -458,7 +462,8 @@ int gemv_i4g32_splitk_geglu_launch(const float *gu, const uint8_t *wp, const uin
 int gemv_i4g32_addnorm_launch(const float *res, const float *delta, int n, const float *w, float eps, float *res_out,
                               const uint8_t *wp, const uint16_t *sc, float *y, int N, int K, hipStream_t st) {
     const GemvPre pre{res, delta, w, res_out, n, eps};
-    if (N >= 8192) return launch_mfma<1, 2, 8, 1, 4, 2048, 2>(nullptr, wp, sc, y, N, K, st, 1, pre);
+    // many rows: workgroups of 16 waves, so that a compute unit forms the activation vector once, not four times
+    if (N >= 8192) return launch_mfma<1, 2, 8, 4, 4, 2048, 2>(nullptr, wp, sc, y, N, K, st, 1, pre);
     return launch_mfma<1, 4, 4, 1, 4, 2048, 2>(nullptr, wp, sc, y, N, K, st, 1, pre);
 }
 
