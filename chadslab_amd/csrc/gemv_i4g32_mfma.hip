@@ -65,7 +65,8 @@ struct GemvCfg {
     static constexpr int XI = (MPASS * (KC / 8) + T - 1) / T;  // 16-byte activation pieces per thread per pass
 };
 
-// waves_per_eu(4): at most 128 VGPRs, which also makes the compiler pick the MFMA form that writes VGPRs.
+// waves_per_eu(4): at most 128 VGPRs, which also makes the compiler pick the MFMA form that writes VGPRs.  The
+// variants for 5 to 8 activation rows with 16 steps per wave need a few more (they spilled at 128): 3 waves, 168.
 // XM: how the activation vector comes about (M = 1 for the modes other than 0).
 //   0  given: x bf16 [M,K].
 //   1  GeGLU folded in: x[k] = bf16( gelu_tanh(gu[k]) * gu[K + k] ) from gu fp32 [2K] (`x` points at gu) - a gated FFN's
@@ -81,7 +82,7 @@ struct GemvPre {
 };
 
 template <int MT, int HP, int S, int RBW, int D, int KC, int XM = 0>
-__global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) void gemv_i4g32_mfma_kernel(
+__global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((MT >= 5 && S == 16) ? 3 : 4))) void gemv_i4g32_mfma_kernel(
     const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
     float *__restrict__ y, int N, int K, int kspan, int pv, GemvPre pre) {
     constexpr bool XG = (XM == 1), XN = (XM == 2);
