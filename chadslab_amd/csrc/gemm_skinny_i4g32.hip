@@ -259,13 +259,17 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
         }
 }
 
-// groups: [E] gate, [E] up, [E] down descriptors as the router writes them.
-// grid: x = N tiles, y = expert * mtiles + token tile, z = K split (MODE 0 only).
+// groups: [E] gate, [E] up, [E] down descriptors as the router writes them; tiles: the token tiles that exist
+// (expert | tile << 16, -1 past the last), also from the router, fullest first.
+// grid: x = N tiles, y = entry of the tile list, z = K split (MODE 0 only).
 template <int MODE>
-__global__ __launch_bounds__(256, SK_WGS_PER_CU) void gemm_skinny_i4g32_kernel(const GemmGroup *__restrict__ groups, int E, int N, int K,
-                                                                  int kspan, int mtiles, size_t ysplit_stride) {
+__global__ __launch_bounds__(256, SK_WGS_PER_CU) void gemm_skinny_i4g32_kernel(const GemmGroup *__restrict__ groups,
+                                                                  const int32_t *__restrict__ tiles, int E, int N, int K,
+                                                                  int kspan, size_t ysplit_stride) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const int g = blockIdx.y / mtiles, mt = blockIdx.y % mtiles;
+    const int tile = tiles[blockIdx.y];
+    if (tile < 0) return;
+    const int g = tile & 0xFFFF, mt = tile >> 16;
     const GemmGroup ga = groups[MODE == 1 ? g : 2 * E + g];
     const int M = ga.M, m0 = mt * SK_MT;
     if (m0 >= M) return;
@@ -295,27 +299,30 @@ __global__ __launch_bounds__(256, SK_WGS_PER_CU) void gemm_skinny_i4g32_kernel(c
 bool gemm_skinny_ok(int H, int F) { return H % 256 == 0 && F % 256 == 0; }
 
 template <int MODE>
-static int skinny_launch(const GemmGroup *groups, int E, int mtiles, int ntiles, int N, int K, int ksplit, size_t ystride,
-                         hipStream_t st) {
+static int skinny_launch(const GemmGroup *groups, const int32_t *tiles, int mtiles, int E, int ntiles, int N, int K, int ksplit,
+                         size_t ystride, hipStream_t st) {
     static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
     if (!attr_set.load(std::memory_order_acquire)) {
         CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_skinny_i4g32_kernel<MODE>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS));
         attr_set.store(true, std::memory_order_release);
     }
-    hipLaunchKernelGGL((gemm_skinny_i4g32_kernel<MODE>), dim3(ntiles, E * mtiles, ksplit), dim3(256), SK_LDS, st,
-                       groups, E, N, K, K / ksplit, mtiles, ystride);
+    hipLaunchKernelGGL((gemm_skinny_i4g32_kernel<MODE>), dim3(ntiles, mtiles, ksplit), dim3(256), SK_LDS, st, groups, tiles, E, N, K,
+                       K / ksplit, ystride);
     return hip_check(hipGetLastError(), "gemm_skinny launch");
 }
 
+int gemm_skinny_tile_rows() { return SK_MT; }
+
 // gate/up with the SiLU epilogue: h[P,F] bf16 (through the down descriptors' x pointers)
-int gemm_skinny_gateup(const GemmGroup *groups, int E, int m_max, int F, int H, hipStream_t st) {
-    return skinny_launch<1>(groups, E, (m_max + SK_MT - 1) / SK_MT, F / 128, F, H, 1, 0, st);
+int gemm_skinny_gateup(const GemmGroup *groups, const int32_t *tiles, int ntiles, int E, int F, int H, hipStream_t st) {
+    return skinny_launch<1>(groups, tiles, ntiles, E, F / 128, F, H, 1, 0, st);
 }
 
 // down: fp32 parts [ksplit][P,H]
-int gemm_skinny_down(const GemmGroup *groups, int E, int m_max, int H, int F, int ksplit, size_t ysplit_stride, hipStream_t st) {
-    return skinny_launch<0>(groups, E, (m_max + SK_MT - 1) / SK_MT, H / 256, H, F, ksplit, ysplit_stride, st);
+int gemm_skinny_down(const GemmGroup *groups, const int32_t *tiles, int ntiles, int E, int H, int F, int ksplit, size_t ysplit_stride,
+                     hipStream_t st) {
+    return skinny_launch<0>(groups, tiles, ntiles, E, H / 256, H, F, ksplit, ysplit_stride, st);
 }
 
 }  // namespace chadq

@@ -26,6 +26,7 @@ struct MoeWs {  // workspace carved up on the host
     int32_t *tok;        // [P] token of the sorted row
     int32_t *cnt;        // [E] rows per expert, then [E] offsets
     GemmGroup *groups;   // [3*E] gate, up, down
+    int32_t *tiles;      // token tiles of the expert GEMMs: expert | tile << 16, -1 past the last one
     uint16_t *xs;        // [P,H] gathered activations (bf16)
     float *g, *u;        // [P,F]
     uint16_t *h;         // [P,F] bf16
@@ -36,8 +37,10 @@ constexpr int MOE_KSPLIT = 4;
 
 int gemm_i4g32_grouped(const GemmGroup *groups, int ngroups, int m_max, int N, int K, bool out_f32, hipStream_t st);
 bool gemm_skinny_ok(int H, int F);
-int gemm_skinny_gateup(const GemmGroup *groups, int E, int m_max, int F, int H, hipStream_t st);
-int gemm_skinny_down(const GemmGroup *groups, int E, int m_max, int H, int F, int ksplit, size_t ysplit_stride, hipStream_t st);
+int gemm_skinny_tile_rows();
+int gemm_skinny_gateup(const GemmGroup *groups, const int32_t *tiles, int ntiles, int E, int F, int H, hipStream_t st);
+int gemm_skinny_down(const GemmGroup *groups, const int32_t *tiles, int ntiles, int E, int H, int F, int ksplit, size_t ysplit_stride,
+                     hipStream_t st);
 
 // One workgroup.  Phase 1: softmax + top-k per token.  Phase 2: stable counting sort of the pairs by expert.
 // Phase 3: descriptors.  idx/w may be the caller's arrays (chadq_moe_route) with everything else null.
@@ -135,9 +138,24 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
     }
 }
 
-// xs[row] = x[tok[row]]; one 16-byte piece per thread
+// xs[row] = x[tok[row]]; one 16-byte piece per thread.  Beside the copy, one thread of the last workgroup lists the
+// token tiles of the expert GEMMs (expert | tile << 16, then -1), the fullest first: they take longest, and no
+// workgroup is launched for a tile that does not exist except at the end of the grid.
 __global__ __launch_bounds__(256) void moe_gather_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ tok,
-                                                         uint16_t *__restrict__ xs, int P, int H) {
+                                                         uint16_t *__restrict__ xs, int P, int H, const int32_t *__restrict__ cnt,
+                                                         int32_t *__restrict__ tiles, int E, int tile_rows, int ntiles_max) {
+    if (tiles && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+        int n = 0;
+        for (int lim = tile_rows; lim > 0 && n < ntiles_max; lim -= 32)  // classes of 32 rows: (lim - 32, lim]
+            for (int e = 0; e < E; ++e) {
+                const int m = cnt[e];
+                for (int mt = 0; mt * tile_rows < m; ++mt) {
+                    const int rows = min(m - mt * tile_rows, tile_rows);
+                    if (rows <= lim && rows > lim - 32 && n < ntiles_max) tiles[n++] = e | (mt << 16);
+                }
+            }
+        for (; n < ntiles_max; ++n) tiles[n] = -1;
+    }
     const int pieces = H / 8;
     const int64_t total = (int64_t)P * pieces, stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
@@ -199,6 +217,7 @@ static size_t moe_layout(uint8_t *base, int T, int H, int F, int E, int top_k, M
     w.tok = (int32_t *)take(P * 4);
     w.cnt = (int32_t *)take((size_t)2 * E * 4);
     w.groups = (GemmGroup *)take((size_t)3 * E * sizeof(GemmGroup));
+    w.tiles = (int32_t *)take(((size_t)E + P / 32 + 1) * 4);
     w.xs = (uint16_t *)take(P * H * 2);
     w.g = (float *)take(P * F * 4);
     w.u = (float *)take(P * F * 4);
@@ -232,8 +251,9 @@ int moe_ffn_i4g32_launch(const uint16_t *x, const float *logits, const chadq_moe
     }
     const int P = T * top_k;
     const int m_max = P < T ? P : T;  // an expert gets a token at most once
+    const int tile_rows = gemm_skinny_tile_rows(), ntiles = E + P / tile_rows;  // sum over experts of ceil(rows / tile_rows) <= this
     hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(T * top_k <= 1024 ? 256 : 1024), 0, st, logits, ws.idx, ws.w, T, E, top_k, renorm, ws, ex, H, F);
-    hipLaunchKernelGGL(moe_gather_kernel, dim3(512), dim3(256), 0, st, x, ws.tok, ws.xs, P, H);
+    hipLaunchKernelGGL(moe_gather_kernel, dim3(512), dim3(256), 0, st, x, ws.tok, ws.xs, P, H, ws.cnt, ws.tiles, E, tile_rows, ntiles);
     int rc = hip_check(hipGetLastError(), "moe route/gather launch");
     if (rc) return rc;
     int nsplit = 1;
@@ -242,10 +262,10 @@ int moe_ffn_i4g32_launch(const uint16_t *x, const float *logits, const chadq_moe
         aligned = aligned && aligned16(experts[e].wg) && aligned16(experts[e].sg) && aligned16(experts[e].wu) &&
                   aligned16(experts[e].su) && aligned16(experts[e].wd) && aligned16(experts[e].sd);
     if (aligned && gemm_skinny_ok(H, F)) {
-        rc = gemm_skinny_gateup(ws.groups, E, m_max, F, H, st);  // h = bf16(silu(gate) * up), [P,F]
+        rc = gemm_skinny_gateup(ws.groups, ws.tiles, ntiles, E, F, H, st);  // h = bf16(silu(gate) * up), [P,F]
         if (rc) return rc;
         nsplit = (F % (256 * MOE_KSPLIT) == 0) ? MOE_KSPLIT : 1;
-        rc = gemm_skinny_down(ws.groups, E, m_max, H, F, nsplit, (size_t)P * H, st);  // fp32 parts [nsplit][P,H]
+        rc = gemm_skinny_down(ws.groups, ws.tiles, ntiles, E, H, F, nsplit, (size_t)P * H, st);  // fp32 parts [nsplit][P,H]
         if (rc) return rc;
     } else {
         rc = gemm_i4g32_grouped(ws.groups, 2 * E, m_max, F, H, true, st);  // gate and up: fp32 [P,F] each
