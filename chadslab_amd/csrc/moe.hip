@@ -48,7 +48,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
                                                          float *__restrict__ w, int T, int E, int top_k, int renorm,
                                                          MoeWs ws, MoeExperts ex, int H, int F) {
     __shared__ int s_base[MOE_MAX_E];   // rows of expert e seen so far
-    __shared__ int s_wave[16];          // per-wave counts of the current expert in the current chunk
+    __shared__ int s_cnt[16][MOE_MAX_E];  // per-wave counts of every expert in the current chunk
     __shared__ int s_off[MOE_MAX_E + 1];
     // expert and rank of every pair stay in LDS between the phases when they fit (a global write followed by a read
     // from other threads costs a memory round trip per phase)
@@ -91,24 +91,26 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
     for (int c0 = 0; c0 < P; c0 += B) {
         const int p = c0 + tid;
         const int e_mine = p < P ? (in_lds ? (int)s_e[p] : idx[p]) : -1;
-        int rank = 0;
+        // every wave counts all experts by itself (one ballot each, no barrier), the counts meet in LDS once per chunk
+        int below = 0;
         for (int e = 0; e < E; ++e) {
-            const bool flag = (e_mine == e);
-            const unsigned long long m = __ballot(flag);
-            const int below = __popcll(m & ((1ull << lane) - 1ull));
-            if (lane == 0) s_wave[wave] = __popcll(m);
-            __syncthreads();
-            int woff = 0, total = 0;
-            for (int i = 0; i < nw; ++i) {
-                const int c = s_wave[i];
-                woff += (i < wave) ? c : 0;
-                total += c;
-            }
-            if (flag) rank = s_base[e] + woff + below;
-            __syncthreads();
-            if (tid == 0) s_base[e] += total;
-            __syncthreads();
+            const unsigned long long m = __ballot(e_mine == e);
+            if (e_mine == e) below = __popcll(m & ((1ull << lane) - 1ull));
+            if (lane == 0) s_cnt[wave][e] = __popcll(m);
         }
+        __syncthreads();
+        int rank = 0;
+        if (e_mine >= 0) {
+            rank = s_base[e_mine] + below;
+            for (int i = 0; i < wave; ++i) rank += s_cnt[i][e_mine];
+        }
+        __syncthreads();
+        if (tid < E) {
+            int total = 0;
+            for (int i = 0; i < nw; ++i) total += s_cnt[i][tid];
+            s_base[tid] += total;
+        }
+        __syncthreads();
         if (p < P) {  // rank inside its expert for now
             if (in_lds) s_r[p] = (uint16_t)rank;
             else ws.pos[p] = rank;
