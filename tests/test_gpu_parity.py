@@ -333,6 +333,21 @@ def test_moe_ffn(ops, t, h, f, e, top_k):
     assert np.array_equal(yp, y[perm])
 
 
+def test_moe_ffn_empty_experts_and_one_crowded_expert(ops):
+    # experts 2..7 get nothing, expert 0 gets every token (three token tiles of 96), expert 1 the second choice of most
+    t, h, f, e = 250, 256, 512, 8
+    host, dev = _experts(90, e, h, f)
+    r = rng(91)
+    xb = O.f32_to_bf16(r.standard_normal((t, h)).astype(np.float32))
+    logits = r.standard_normal((t, e)).astype(np.float32)
+    logits[:, 0] += 30.0
+    logits[:, 1] += 15.0
+    logits[:7, 1] -= 40.0  # a few tokens take some other expert second: tiles of very few rows
+    y = O.bf16_to_f32(bits(ops.moe_ffn(bf16_tensor(xb), torch.from_numpy(logits).to(DEV), dev, top_k=2, renorm=True)))
+    ref = O.bf16_to_f32(O.moe_qffn(xb, logits, host, 2, True))
+    assert np.isfinite(y).all() and O.rel_l2(y, ref) <= TOL_BF16
+
+
 def test_moe_config3_full_size(ops):
     t, h, f, e = 256, 4096, 14336, 8
     host, dev = _experts(1003, e, h, f)
