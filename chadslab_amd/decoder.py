@@ -217,6 +217,20 @@ class QuantDecoder:
         torch.cuda.synchronize()
         self.graph = g
 
+    def feed(self, tokens, pos: int = 0) -> int:
+        """Runs the step over a given token sequence starting at position `pos` (the prompt, one token at a time: there
+        is no batched prefill here), filling the caches; returns the token the model proposes after the last one."""
+        self.pos.fill_(pos)
+        for t in tokens:
+            self.token.fill_(int(t))  # overrides the token the previous step proposed
+            if self.sampling is not None:
+                self.u.uniform_(0.0, 1.0, generator=self.rng)
+            if self.graph is not None:
+                self.graph.replay()
+            else:
+                self.step()
+        return int(self.token.item())
+
     def generate(self, first_token: int, pos: int, n: int) -> List[int]:
         """Decodes n tokens starting from `first_token` at position `pos` (the cache holds pos rows): greedy, or sampled
         as set_sampling() says."""

@@ -432,6 +432,20 @@ def test_decoder_sampling_eager_and_graph_draw_the_same_tokens():
     assert all(0 <= t < cfg.vocab for t in sampled) and sampled != greedy
 
 
+def test_decoder_feed_then_generate_continues_the_same_sequence():
+    from chadslab_amd.decoder import DecoderConfig, QuantDecoder
+
+    cfg = DecoderConfig(n_layers=2, d=512, hq=4, dh=64, ffn=1024, vocab=1000, max_ctx=256)
+    m = _upload(_model(47, cfg))
+    a = QuantDecoder(cfg, m, DEV)
+    seq = a.generate(5, 0, 12)           # 5 -> seq[0] -> seq[1] ...
+    b = QuantDecoder(cfg, m, DEV)
+    b.capture()
+    nxt = b.feed([5] + seq[:6], 0)       # teacher-forced over the first seven tokens
+    assert nxt == seq[6] and int(b.pos.item()) == 7
+    assert b.generate(nxt, 7, 5) == seq[7:12]
+
+
 def test_decoder_step_odd_layer_count_graph_replay():
     from chadslab_amd.decoder import DecoderConfig
 
