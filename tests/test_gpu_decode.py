@@ -254,6 +254,29 @@ def test_rope_table_matches_the_rotation(lib):
     assert np.abs(t[..., 0] - np.cos(ang)).max() < 2e-4 and np.abs(t[..., 1] - np.sin(ang)).max() < 2e-4
 
 
+def test_attention_random_shapes(lib):
+    r = rng(777)
+    for _ in range(14):
+        hq = int(r.integers(1, 9))
+        dh = int(r.choice([16, 32, 48, 64, 96, 128, 160, 256]))
+        max_ctx = int(r.integers(40, 3000))
+        pos = int(r.integers(0, max_ctx))
+        test_attn_decode_mqa_fused_equals_rope_write_attend(lib, hq, dh, pos, max_ctx)
+        test_attn_decode_mqa(lib, hq, dh, pos, max_ctx)
+
+
+def test_gemv_addnorm_and_geglu_random_shapes(lib):
+    r = rng(778)
+    for _ in range(10):
+        k = 256 * int(r.integers(1, 9))
+        n = int(r.integers(1, 3000)) if r.random() < 0.7 else int(r.integers(8192, 9000))
+        test_gemv_addnorm_equals_norm_then_gemv(lib, n, k, int(r.integers(0, 5)))
+    for _ in range(6):
+        ksplit = int(r.choice([1, 2, 4]))
+        k = 4096 * ksplit * int(r.integers(1, 3))
+        test_gemv_splitk_geglu_equals_geglu_then_gemv(lib, int(r.integers(1, 1200)), k, ksplit)
+
+
 @pytest.mark.parametrize("F", [1, 255, 16384])
 def test_geglu(lib, F):
     gu = (rng(F).standard_normal(2 * F) * 3).astype(np.float32)

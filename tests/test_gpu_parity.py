@@ -206,6 +206,39 @@ def test_gemv_int8_integer_exact(ops):
     assert np.array_equal(y.astype(np.int64), x.astype(np.int64) @ w.astype(np.int64).T)
 
 
+# ------------------------------------------------------------------ seeded random shapes (ragged edges of every kind)
+def test_random_shapes_int4_gemv_and_gemm(ops):
+    r = rng(4242)
+    for case in range(36):
+        m = int(r.choice([1, 2, 3, 4, 5, 7, 8, 9, 16, 17, 40, 130]))
+        n = int(r.integers(1, 700)) if case % 3 else int(r.integers(8192, 9500))
+        k = 32 * int(r.integers(1, 70))
+        if n >= 8192:
+            k = 32 * int(r.integers(1, 20))  # keep the float64 reference quick
+        packed, s, xb, qw = i4_case(5000 + case, m, n, k)
+        ref = O.qgemm_int4g32_f64(xb, packed, s)
+        if m <= 16:
+            y = ops.qgemv(bf16_tensor(xb), qw).cpu().numpy()
+            assert y.shape == (m, n) and np.isfinite(y).all() and O.rel_l2(y, ref) <= TOL_F32, ("gemv", m, n, k)
+        yb = O.bf16_to_f32(bits(ops.qgemm(bf16_tensor(xb), qw)))
+        assert yb.shape == (m, n) and np.isfinite(yb).all() and O.rel_l2(yb, ref) <= TOL_BF16, ("gemm", m, n, k)
+
+
+def test_random_shapes_int8(ops):
+    r = rng(4243)
+    for case in range(16):
+        m = int(r.choice([1, 3, 8, 33, 129]))
+        n = int(r.integers(1, 600))
+        k = 16 * int(r.integers(1, 90))
+        x, w, s, q8 = i8_case(6000 + case, m, n, k)
+        xb = O.f32_to_bf16(x)
+        yb = O.bf16_to_f32(bits(ops.qgemm(bf16_tensor(xb), q8)))
+        assert O.rel_l2(yb, O.qgemm_int8_f64(xb, w, s)) <= TOL_BF16, ("gemm8", m, n, k)
+        y1 = ops.qgemv(torch.from_numpy(x[:1]).to(DEV), q8).cpu().numpy()
+        ref1 = (x[:1].astype(np.float64) @ (w.astype(np.float64) * s[:, None].astype(np.float64)).T)
+        assert O.rel_l2(y1, ref1) <= TOL_F32, ("gemv8", n, k)
+
+
 # ------------------------------------------------------------------ prefill GEMM (config 2)
 @pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (1, 64, 128), (37, 100, 96), (130, 70, 288), (5, 33, 32), (128, 64, 256), (200, 192, 1056)])
 def test_gemm_int4(ops, m, n, k):
@@ -346,6 +379,24 @@ def test_moe_ffn_empty_experts_and_one_crowded_expert(ops):
     y = O.bf16_to_f32(bits(ops.moe_ffn(bf16_tensor(xb), torch.from_numpy(logits).to(DEV), dev, top_k=2, renorm=True)))
     ref = O.bf16_to_f32(O.moe_qffn(xb, logits, host, 2, True))
     assert np.isfinite(y).all() and O.rel_l2(y, ref) <= TOL_BF16
+
+
+def test_moe_ffn_random_shapes(ops):
+    r = rng(4244)
+    for case in range(8):
+        e = int(r.integers(1, 9))
+        top_k = int(r.integers(1, min(e, 4) + 1))
+        t = int(r.integers(1, 300))
+        if case % 2:  # shapes the expert kernel takes (multiples of 256) / shapes that go the general way
+            h, f = 256 * int(r.integers(1, 4)), 256 * int(r.integers(1, 4))
+        else:
+            h, f = 32 * int(r.integers(1, 12)), 32 * int(r.integers(1, 12))
+        host, dev = _experts(7000 + case, e, h, f)
+        xb = O.f32_to_bf16(r.standard_normal((t, h)).astype(np.float32))
+        logits = r.standard_normal((t, e)).astype(np.float32)
+        y = O.bf16_to_f32(bits(ops.moe_ffn(bf16_tensor(xb), torch.from_numpy(logits).to(DEV), dev, top_k=top_k, renorm=bool(case & 2))))
+        ref = O.bf16_to_f32(O.moe_qffn(xb, logits, host, top_k, bool(case & 2)))
+        assert np.isfinite(y).all() and O.rel_l2(y, ref) <= TOL_BF16, (t, h, f, e, top_k)
 
 
 def test_moe_config3_full_size(ops):
