@@ -164,6 +164,22 @@ def main():
         extras["gemv_i4g32"]["M1_same_buffer_every_step"] = {
             "us": round(us_hot, 3), "GBps": round(gemv_bytes(1) / us_hot * 1e-3, 1),
             "note": "weights served by the 256 MB last-level cache, not HBM; not a roofline figure"}
+        # what this machine delivers for a cold read of the same number of bytes with the same access shape and no
+        # arithmetic: the practical ceiling next to which the GEMV's time should be read
+        lib = _lib.load()
+        nread = gemv_bytes(1) // 16384 * 16384
+        flat = [torch.empty(nread, dtype=torch.uint8, device=dev).fill_(i + 1) for i in range(N_COPIES)]
+        pout = torch.empty(nread // 16384, dtype=torch.int32, device=dev)
+
+        def probe(i):
+            _lib.check(lib.chadq_probe_read(flat[i % N_COPIES].data_ptr(), nread, pout.data_ptr(),
+                                            torch.cuda.current_stream().cuda_stream), "chadq_probe_read")
+
+        us_rd, _ = run_steps(probe, *n_side)
+        extras["gemv_i4g32"]["cold_read_same_bytes"] = {
+            "us": round(us_rd, 3), "GBps": round(nread / us_rd * 1e-3, 1), "bytes": int(nread),
+            "note": "loads only (chadq_probe_read), rotating buffers: the machine's ceiling for a read of this size"}
+        del flat, pout
     del copies
 
     if "int8" in want:
@@ -196,6 +212,14 @@ def main():
             usg, _ = run_steps(lambda i: ops.qgemm(x2, qw, out=y2), *n_gemm)
             extras[name] = {"us": round(usg, 3), "TFLOPs": round(flop / usg * 1e-6, 1),
                             "frac_bf16_mfma_peak": round(flop / usg * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+
+        # context: the vendor library's plain bf16 GEMM (no dequantisation) on the same shape, through torch.matmul
+        wb16 = torch.randn(N2, K2, device=dev).to(torch.bfloat16)
+        yt = torch.empty(M2, N2, dtype=torch.bfloat16, device=dev)
+        ust, _ = run_steps(lambda i: torch.matmul(x2, wb16.t(), out=yt), *n_gemm)
+        extras["gemm_bf16_library_same_shape"] = {"us": round(ust, 3), "TFLOPs": round(flop / ust * 1e-6, 1),
+                                                  "note": "torch.matmul on bf16 weights (hipBLASLt/rocBLAS): context, not this build's kernel"}
+        del wb16, yt
 
         # the kernel's asymptote at a larger M (not a benchmark config: extra, labelled as such)
         M2b = 4096

@@ -44,6 +44,7 @@ SIGNATURES = {
                                             c_void_p]),
     "chadq_geglu_bf16": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     "chadq_argmax_f32": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "chadq_probe_read": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "chadq_sample_topk_f32": (c_int, [c_void_p, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
 }
 

@@ -93,6 +93,19 @@ def test_dequant_exact(ops):
     assert np.array_equal(ops.dequantize(q8).cpu().numpy(), O.dequant_int8(w, s8))
 
 
+def test_probe_read_reads_every_byte(ops):
+    from chadslab_amd import _lib
+
+    lib = _lib.load()
+    n = 5 * 16384 + 100  # the tail that does not fill 16 KiB is left alone
+    data = rng(11).integers(0, 256, n, dtype=np.uint8)
+    t = torch.from_numpy(data).to(DEV)
+    out = torch.zeros(n // 16384, dtype=torch.int32, device=DEV)
+    _lib.check(lib.chadq_probe_read(t.data_ptr(), n, out.data_ptr(), torch.cuda.current_stream().cuda_stream), "probe")
+    want = np.bitwise_xor.reduce(data[:5 * 16384].view(np.uint32).reshape(5, -1), axis=1)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want)
+
+
 # ------------------------------------------------------------------ golden fixtures
 def test_golden_int4(ops):
     from chadslab_amd import QWeightInt4G32
