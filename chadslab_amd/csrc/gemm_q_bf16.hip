@@ -86,7 +86,7 @@ struct Tile {
     static constexpr int NSLOT = 8;                 // ring: two iterations of four m-blocks
     static constexpr int A_BYTES = NWAVE * NSLOT * SLOT_BYTES;
     // weights and scales of one iteration of one wave: NB x 1 KiB (16 B per lane) + NB x 256 B (a dword per lane)
-    static constexpr int BSLOT_BYTES = NB * 1024 + NB * 256;
+    static constexpr int BSLOT_BYTES = NB * 1024 + 1024;  // + scales: a dword per lane and n-block, or 16 bytes per weight row
     static constexpr int B_OFF = A_BYTES;
     static constexpr int STAGE_BYTES = A_BYTES + NWAVE * BSLOT_BYTES;
     static constexpr int EPI_BYTES = NWAVE * BM * 32 * 4;
@@ -152,6 +152,15 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
         wbase[nb] = (const uint8_t *)wq + (size_t)nc * wrow_bytes;  // row starts; k offsets are added per load
         sbase[nb] = (const uint16_t *)sc + (size_t)nc * G;
     }
+    // Scales, unguarded form: one request per iteration fetches, for each of the tile's 32*NB weight rows (lane -> row),
+    // the aligned 16 bytes = 8 groups = this iteration's 256 k of all four waves; a lane later picks its own group.
+    // (Two requests of 2 bytes per lane, the general form, cost 9 % of the kernel's time: requests, not bytes, count.)
+    constexpr bool SBLK = i4 && !GUARD && NB == 2;
+    const uint16_t *srow_blk = nullptr;
+    if (SBLK) {
+        const int n = n0 + lane;
+        srow_blk = (const uint16_t *)sc + (size_t)(n < N ? n : N - 1) * G;
+    }
     // DMA: LDS position lane*16 inside each 1 KiB block is (row dr, slot dslot); the piece that belongs there is
     // dslot ^ key(row).  Per-lane byte offsets into x are 32-bit (the host checks M*K*2 < 2^32); the k advance
     // per iteration goes into the scalar base.
@@ -193,10 +202,11 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
         for (int nb = 0; nb < NB; ++nb) {
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wbase[nb] + (i4 ? kc / 2 : kc)),
                                              (__attribute__((address_space(3))) void *)(bslot + nb * 1024), 16, 0, 0);
-            if (i4)
+            if (i4 && !SBLK)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(sbase[nb] + (kc >> 5)),
                                                  (__attribute__((address_space(3))) void *)(bslot + NB * 1024 + nb * 256), 2, 0, 0);
         }
+        if (SBLK) dma16_to_lds(srow_blk + it * (TL::KIT / 32), bslot + NB * 1024);
     };
     const uint32_t c_mlo = vgpr_const(0x000F000Fu), c_mhi = vgpr_const(0x00F000F0u), c_magic = vgpr_const(0x64006400u);
     bf16x8 bf[2][TL::T][NB];  // [set][step][n-block]: dequantised weights of one iteration
@@ -209,7 +219,9 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
         for (int nb = 0; nb < NB; ++nb) {
             cq[nb] = *reinterpret_cast<const u32x4 *>(src + nb * 1024 + lane * 16);
             if constexpr (i4) {
-                const float s = live ? f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(src + NB * 1024 + nb * 256 + lane * 4)) : 0.f;
+                const uint16_t sb16 = SBLK ? *reinterpret_cast<const uint16_t *>(src + NB * 1024 + (nb * 32 + nl) * 16 + (2 * wave + kq) * 2)
+                                           : *reinterpret_cast<const uint16_t *>(src + NB * 1024 + nb * 256 + lane * 4);
+                const float s = live ? f16_bits_to_f32(sb16) : 0.f;
                 cs[nb][0] = s;
                 cs[nb][1] = s * 0.0625f;
                 cs[nb][2] = -1032.f * s;
@@ -233,7 +245,7 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
     };
 
     const int iters = (K + TL::KIT - 1) / TL::KIT;
-    constexpr int DPM = TL::DPM, NBL = (i4 ? 2 : 1) * NB, LPI = 4 * DPM + NBL;  // VMEM instructions: m-block, weights, iteration
+    constexpr int DPM = TL::DPM, NBL = SBLK ? NB + 1 : (i4 ? 2 : 1) * NB, LPI = 4 * DPM + NBL;  // VMEM instructions: m-block, weights, iteration
     // Request order (memory returns in order, so "X has landed" is "at most so many younger requests are out"):
     //   prologue   W(0) T(0,0..3) | W(1) T(1,0..3)          W = weights+scales of an iteration, T(i,mb) = m-block
     //   iteration i issues, after consuming m-block mb, the refill T(i+2,mb); W(i+2) goes out right after the
@@ -415,7 +427,11 @@ static int launch_gemm(const uint16_t *x, const void *wq, const typename F::scal
                        const GemmGroup *groups, int ngroups, hipStream_t st) {
     CHADQ_REQUIRE((int64_t)M * K * 2 < ((int64_t)1 << 32), CHADQ_ERR_SHAPE,
                   "gemm: activations of %d x %d exceed the 4 GiB the kernel's 32-bit offsets cover", M, K);
-    if (K % Tile<F, 2>::KIT != 0) return launch_gemm_g<F, 2, true, OUTF32>(x, wq, sc, y, M, N, K, groups, ngroups, st);
+    // the unguarded int4 form fetches scale rows 16 bytes at a time: it needs 16-byte aligned scale rows, which only a
+    // plain launch can check here (a grouped launch's pointers live in device memory)
+    const bool scale_rows_ok = Tile<F, 2>::KL != 32 || (!groups && (reinterpret_cast<uintptr_t>(sc) & 15u) == 0);
+    if (K % Tile<F, 2>::KIT != 0 || !scale_rows_ok)
+        return launch_gemm_g<F, 2, true, OUTF32>(x, wq, sc, y, M, N, K, groups, ngroups, st);
     return launch_gemm_g<F, 2, false, OUTF32>(x, wq, sc, y, M, N, K, groups, ngroups, st);
 }
 
