@@ -7,8 +7,9 @@
 // makes both operands private to a wave:
 //   * B (weights): lane (n = lane%32, kq = lane/32) owns 16 packed bytes of output row n per iteration, which
 //     is 32 k (int4, exactly one scale group) or 16 k (int8).  They arrive by direct global->LDS load in a
-//     wave-private slot, the same lane reads them back, dequantises them in registers (fp16 magic numbers,
-//     one fp32 FMA per element, RNE to bf16) and feeds them to the MFMA.  No other lane ever needs them.
+//     wave-private slot (fetched so that the two pieces of a row come from neighbouring lanes: one 32-byte
+//     request), the owning lane reads them back, dequantises them in registers (fp16 magic numbers, one fp32 FMA
+//     per element, RNE to bf16) and feeds them to the MFMA.  No other wave ever needs them.
 //   * A (activations): the wave moves its own 128 x KW slice into a wave-private, double-buffered LDS tile with
 //     direct global->LDS loads (global_load_lds_dwordx4: 8 rows x 128 B per instruction, no VGPR round trip),
 //     purely to turn row-major memory into MFMA fragments.  16-byte pieces are XOR-swizzled by row so that
@@ -142,15 +143,18 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
-    // weight rows of this lane (clamped so that loads stay in bounds; results for n >= N are never stored)
+    // Weight rows (clamped so that loads stay in bounds; results for n >= N are never stored).  The weight request of
+    // n-block nb is issued with lane l fetching piece l % 2 of row l / 2, so that the two 16-byte pieces of a row come
+    // from neighbouring lanes (one 32-byte request, not two of 16); lane (nl, kq) reads its operand back from LDS
+    // position 2 * nl + kq.  Scales in the general form stay one 2-byte request per lane (nl, kq).
+    const int wl_row = lane >> 1, wl_kq = lane & 1;
     const uint8_t *wbase[NB];
     const uint16_t *sbase[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-        const int n = n0 + nb * 32 + nl;
-        const int nc = n < N ? n : N - 1;
-        wbase[nb] = (const uint8_t *)wq + (size_t)nc * wrow_bytes;  // row starts; k offsets are added per load
-        sbase[nb] = (const uint16_t *)sc + (size_t)nc * G;
+        const int nw = n0 + nb * 32 + wl_row, n = n0 + nb * 32 + nl;
+        wbase[nb] = (const uint8_t *)wq + (size_t)(nw < N ? nw : N - 1) * wrow_bytes;  // row starts; k offsets are added per load
+        sbase[nb] = (const uint16_t *)sc + (size_t)(n < N ? n : N - 1) * G;
     }
     // Scales, unguarded form: one request per iteration fetches, for each of the tile's 32*NB weight rows (lane -> row),
     // the aligned 16 bytes = 8 groups = this iteration's 256 k of all four waves; a lane later picks its own group.
@@ -196,11 +200,13 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
     // access a DMA, the explicit counts below are the only waits on vector memory in the loop.
     uint8_t *bslot = lds + TL::B_OFF + wave * TL::BSLOT_BYTES;
     auto issue_b = [&](int it) {
-        const int kw = it * TL::KIT + wave * TL::KW + kq * TL::KL;  // first k of this lane's 16 bytes
+        const int kw = it * TL::KIT + wave * TL::KW + kq * TL::KL;  // first k of the 16 bytes lane (nl, kq) will use
         const int kc = (!GUARD || kw < K) ? kw : 0;                   // past K: the row start, zeroed on use
+        const int kww = it * TL::KIT + wave * TL::KW + wl_kq * TL::KL;  // first k of the 16 bytes this lane fetches
+        const int kcw = (!GUARD || kww < K) ? kww : 0;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wbase[nb] + (i4 ? kc / 2 : kc)),
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wbase[nb] + (i4 ? kcw / 2 : kcw)),
                                              (__attribute__((address_space(3))) void *)(bslot + nb * 1024), 16, 0, 0);
             if (i4 && !SBLK)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(sbase[nb] + (kc >> 5)),
@@ -217,7 +223,7 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
         const uint8_t *src = bslot;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-            cq[nb] = *reinterpret_cast<const u32x4 *>(src + nb * 1024 + lane * 16);
+            cq[nb] = *reinterpret_cast<const u32x4 *>(src + nb * 1024 + (2 * nl + kq) * 16);
             if constexpr (i4) {
                 const uint16_t sb16 = SBLK ? *reinterpret_cast<const uint16_t *>(src + NB * 1024 + (nb * 32 + nl) * 16 + (2 * wave + kq) * 2)
                                            : *reinterpret_cast<const uint16_t *>(src + NB * 1024 + nb * 256 + lane * 4);
