@@ -244,6 +244,7 @@ def main():
         experts = [(mk(F3, H3), mk(F3, H3), mk(H3, F3)) for _ in range(E3)]
         x3 = torch.randn(T3, H3, device=dev, generator=g3).to(torch.bfloat16)
         z3 = torch.randn(T3, E3, device=dev, generator=g3)
+        torch.cuda.synchronize()  # the inputs were generated on the default stream
         with torch.cuda.stream(stream):
             for _ in range(3):
                 ops.moe_ffn(x3, z3, experts)
@@ -270,6 +271,7 @@ def main():
 
         cfg4 = DecoderConfig(max_ctx=4096)
         w4 = random_weights(cfg4, 1004, dev)
+        torch.cuda.synchronize()  # the weights were generated on the default stream
         with torch.cuda.stream(stream):
             dec = QuantDecoder(cfg4, w4, dev)
             for li in range(cfg4.n_layers):
