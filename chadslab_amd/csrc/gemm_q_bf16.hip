@@ -86,8 +86,9 @@ struct Tile {
     static constexpr int SLOT_BYTES = 32 * ROWB;    // one m-block of one iteration
     static constexpr int NSLOT = 8;                 // ring: two iterations of four m-blocks
     static constexpr int A_BYTES = NWAVE * NSLOT * SLOT_BYTES;
-    // weights and scales of one iteration of one wave: NB x 1 KiB (16 B per lane) + NB x 256 B (a dword per lane)
-    static constexpr int BSLOT_BYTES = NB * 1024 + 1024;  // + scales: a dword per lane and n-block, or 16 bytes per weight row
+    // weights and scales of one iteration of one wave: NB x 1 KiB of weights (16 B per lane) + 1 KiB for the scales
+    // (general form: 2 bytes in a 4-byte place per lane and n-block; unguarded int4 form: 16 bytes per weight row)
+    static constexpr int BSLOT_BYTES = NB * 1024 + 1024;
     static constexpr int B_OFF = A_BYTES;
     static constexpr int STAGE_BYTES = A_BYTES + NWAVE * BSLOT_BYTES;
     static constexpr int EPI_BYTES = NWAVE * BM * 32 * 4;
@@ -195,9 +196,9 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
                                              (__attribute__((address_space(3))) void *)(dst + q * 1024), 16, 0, 0);
         }
     };
-    // Weights take the same road: lane (nl, kq) DMAs its 16 packed bytes (and, for int4, its group's scale as
-    // one dword) into a wave-private slot and reads them back itself one iteration later.  With every global
-    // access a DMA, the explicit counts below are the only waits on vector memory in the loop.
+    // Weights take the same road: a lane DMAs 16 packed bytes (and, for int4 in the general form, lane (nl, kq) its
+    // group's scale) into a wave-private slot; lane (nl, kq) reads its operand back one iteration later.  With every
+    // global access a DMA, the explicit counts below are the only waits on vector memory in the loop.
     uint8_t *bslot = lds + TL::B_OFF + wave * TL::BSLOT_BYTES;
     auto issue_b = [&](int it) {
         const int kw = it * TL::KIT + wave * TL::KW + kq * TL::KL;  // first k of the 16 bytes lane (nl, kq) will use
