@@ -58,31 +58,60 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
     const int tid = threadIdx.x, B = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = B >> 6;
     const bool in_lds = (T * top_k <= LP) && ws.pos;
     if (tid < MOE_MAX_E) s_base[tid] = 0;
+    // the expert's six pointers are asked for now (they sit in the kernel-argument buffer, indexed per lane) and used at
+    // the very end
+    const void *e_wg = nullptr, *e_sg = nullptr, *e_wu = nullptr, *e_su = nullptr, *e_wd = nullptr, *e_sd = nullptr;
+    if (ws.pos && tid < E) {
+        e_wg = ex.wg[tid];
+        e_sg = ex.sg[tid];
+        e_wu = ex.wu[tid];
+        e_su = ex.su[tid];
+        e_wd = ex.wd[tid];
+        e_sd = ex.sd[tid];
+    }
 
     for (int t = tid; t < T; t += B) {
+        // the token's logits go to registers once (every load in flight together); places past E hold -inf and are
+        // never candidates
         const float *z = logits + (size_t)t * E;
-        float mx = z[0];
-        for (int e = 1; e < E; ++e) mx = fmaxf(mx, z[e]);
+        float zr[MOE_MAX_E];
+#pragma unroll
+        for (int e = 0; e < MOE_MAX_E; ++e) zr[e] = (e < E) ? z[e] : -INFINITY;
+        float mx = zr[0];
+#pragma unroll
+        for (int e = 1; e < MOE_MAX_E; ++e)
+            if (e < E) mx = fmaxf(mx, zr[e]);
         float sum = 0.f;
-        for (int e = 0; e < E; ++e) sum += __expf(z[e] - mx);
+#pragma unroll
+        for (int e = 0; e < MOE_MAX_E; ++e)
+            if (e < E) sum += __expf(zr[e] - mx);
+        uint32_t taken = 0;
         int chosen[MOE_MAX_K];
         float pw[MOE_MAX_K], wsum = 0.f;
-        for (int j = 0; j < top_k; ++j) {
-            int best = -1;
-            for (int e = 0; e < E; ++e) {
-                bool taken = false;
-                for (int i = 0; i < j; ++i) taken |= (chosen[i] == e);
-                if (!taken && (best < 0 || z[e] > z[best])) best = e;  // strict >: the lowest index wins ties
+#pragma unroll
+        for (int j = 0; j < MOE_MAX_K; ++j) {
+            if (j < top_k) {
+                int best = -1;
+                float bv = 0.f;
+#pragma unroll
+                for (int e = 0; e < MOE_MAX_E; ++e)
+                    if (e < E && !((taken >> e) & 1u) && (best < 0 || zr[e] > bv)) {  // strict >: the lowest index wins ties
+                        best = e;
+                        bv = zr[e];
+                    }
+                taken |= 1u << best;
+                chosen[j] = best;
+                pw[j] = __expf(bv - mx) / sum;
+                wsum += pw[j];
             }
-            chosen[j] = best;
-            pw[j] = __expf(z[best] - mx) / sum;
-            wsum += pw[j];
         }
-        for (int j = 0; j < top_k; ++j) {
-            idx[(size_t)t * top_k + j] = chosen[j];
-            w[(size_t)t * top_k + j] = renorm ? pw[j] / wsum : pw[j];
-            if (in_lds) s_e[t * top_k + j] = (uint8_t)chosen[j];
-        }
+#pragma unroll
+        for (int j = 0; j < MOE_MAX_K; ++j)
+            if (j < top_k) {
+                idx[(size_t)t * top_k + j] = chosen[j];
+                w[(size_t)t * top_k + j] = renorm ? pw[j] / wsum : pw[j];
+                if (in_lds) s_e[t * top_k + j] = (uint8_t)chosen[j];
+            }
     }
     if (!ws.pos) return;  // routing only
     __syncthreads();      // idx (global) written by this workgroup is visible to it after the barrier
@@ -116,15 +145,15 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
             else ws.pos[p] = rank;
         }
     }
-    if (tid == 0) {
+    if (tid < E) {  // first row of every expert: each of the E threads adds the counts before its own
         int o = 0;
-        for (int e = 0; e < E; ++e) {
-            s_off[e] = o;
-            ws.cnt[e] = s_base[e];
-            ws.cnt[E + e] = o;
-            o += s_base[e];
-        }
-        s_off[E] = o;
+#pragma unroll
+        for (int e = 0; e < MOE_MAX_E; ++e)
+            if (e < tid) o += s_base[e];
+        s_off[tid] = o;
+        ws.cnt[tid] = s_base[tid];
+        ws.cnt[E + tid] = o;
+        if (tid == E - 1) s_off[E] = o + s_base[tid];
     }
     __syncthreads();
     for (int p = tid; p < P; p += B) {
@@ -134,9 +163,9 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
     }
     if (tid < E) {
         const int e = tid, o = s_off[e], m = s_base[e];
-        ws.groups[e] = GemmGroup{ws.xs + (size_t)o * H, ex.wg[e], ex.sg[e], ws.g + (size_t)o * F, m, 0};
-        ws.groups[E + e] = GemmGroup{ws.xs + (size_t)o * H, ex.wu[e], ex.su[e], ws.u + (size_t)o * F, m, 0};
-        ws.groups[2 * E + e] = GemmGroup{ws.h + (size_t)o * F, ex.wd[e], ex.sd[e], ws.yp + (size_t)o * H, m, 0};
+        ws.groups[e] = GemmGroup{ws.xs + (size_t)o * H, e_wg, e_sg, ws.g + (size_t)o * F, m, 0};
+        ws.groups[E + e] = GemmGroup{ws.xs + (size_t)o * H, e_wu, e_su, ws.u + (size_t)o * F, m, 0};
+        ws.groups[2 * E + e] = GemmGroup{ws.h + (size_t)o * F, e_wd, e_sd, ws.yp + (size_t)o * H, m, 0};
     }
 }
 
@@ -254,7 +283,7 @@ int moe_ffn_i4g32_launch(const uint16_t *x, const float *logits, const chadq_moe
     const int P = T * top_k;
     const int m_max = P < T ? P : T;  // an expert gets a token at most once
     const int tile_rows = gemm_skinny_tile_rows(), ntiles = E + P / tile_rows;  // sum over experts of ceil(rows / tile_rows) <= this
-    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(T * top_k <= 1024 ? 256 : 1024), 0, st, logits, ws.idx, ws.w, T, E, top_k, renorm, ws, ex, H, F);
+    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(P <= 256 ? 256 : P <= 512 ? 512 : 1024), 0, st, logits, ws.idx, ws.w, T, E, top_k, renorm, ws, ex, H, F);
     hipLaunchKernelGGL(moe_gather_kernel, dim3(512), dim3(256), 0, st, x, ws.tok, ws.xs, P, H, ws.cnt, ws.tiles, E, tile_rows, ntiles);
     int rc = hip_check(hipGetLastError(), "moe route/gather launch");
     if (rc) return rc;
