@@ -70,8 +70,9 @@ constexpr int SK_WGS_PER_CU = (2 * SK_LDS <= 160 * 1024) ? 2 : 1;
 template <int MODE, int MB>
 __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, const uint8_t *__restrict__ w0,
                                             const uint16_t *__restrict__ s0, const uint8_t *__restrict__ w1,
-                                            const uint16_t *__restrict__ s1, void *__restrict__ yv, int m0, int rows,
-                                            int n0, int N, int K, int kbeg, int kend, uint8_t *lds) {
+                                            const uint16_t *__restrict__ s1, void *__restrict__ yv,
+                                            const int32_t *__restrict__ rowidx, int m0, int rows, int n0, int N, int K,
+                                            int kbeg, int kend, uint8_t *lds) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nl = lane & 31, kq = lane >> 5;
@@ -106,12 +107,15 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
         }
     // activation pieces this lane requests: DMA instruction i of wave w fills LDS bytes (4i + w) * 1024 + 16 * lane
     // of a stage, i.e. row rr = (4i + w) * 8 + lane / 8, slot lane % 8, which holds piece slot ^ (rr & 7).  Rows
-    // past the tile repeat its last row (their results are never stored).
+    // past the tile repeat its last row (their results are never stored).  With a row index (gate/up: the tokens
+    // routed to the expert, in the expert's row order) row m of the tile is row rowidx[m] of x: the activations are
+    // read where they lie, no gathered copy exists.
     const uint16_t *asrc[MB];
 #pragma unroll
     for (int i = 0; i < MB; ++i) {
         const int rr = (4 * i + wave) * 8 + (lane >> 3), rc = rr < rows ? rr : rows - 1;
-        asrc[i] = x + (size_t)(m0 + rc) * K + (((lane & 7) ^ (rr & 7)) << 3);
+        const size_t srow = rowidx ? (size_t)rowidx[m0 + rc] : (size_t)(m0 + rc);
+        asrc[i] = x + srow * K + (((lane & 7) ^ (rr & 7)) << 3);
     }
     // fragment read offsets: row mb*32 + nl, piece kq*4 + j lives in slot (kq*4 + j) ^ (nl & 7)
     uint32_t ard[4];
@@ -260,11 +264,14 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
 }
 
 // groups: [E] gate, [E] up, [E] down descriptors as the router writes them; tiles: the token tiles that exist
-// (expert | tile << 16, -1 past the last), also from the router, fullest first.
+// (expert | tile << 16, -1 past the last), also from the router, fullest first.  MODE 1 with tok != nullptr: the
+// gate/up descriptors' x is the ungathered activation matrix and `pad` the expert's first row in tok, the token of
+// every expert-sorted row.
 // grid: x = N tiles, y = entry of the tile list, z = K split (MODE 0 only).
 template <int MODE>
 __global__ __launch_bounds__(256, SK_WGS_PER_CU) void gemm_skinny_i4g32_kernel(const GemmGroup *__restrict__ groups,
-                                                                  const int32_t *__restrict__ tiles, int E, int N, int K,
+                                                                  const int32_t *__restrict__ tiles,
+                                                                  const int32_t *__restrict__ tok, int E, int N, int K,
                                                                   int kspan, size_t ysplit_stride) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tile = tiles[blockIdx.y];
@@ -289,40 +296,43 @@ __global__ __launch_bounds__(256, SK_WGS_PER_CU) void gemm_skinny_i4g32_kernel(c
         y = reinterpret_cast<float *>(ga.y) + (size_t)blockIdx.z * ysplit_stride;
         n0 = blockIdx.x * 256;
     }
+    const int32_t *rowidx = (MODE == 1 && tok) ? tok + ga.pad : nullptr;
     switch ((rows + 31) >> 5) {
-        case 1: skinny_body<MODE, 1>(ga.x, w0, s0, w1, s1, y, m0, rows, n0, N, K, kbeg, kend, lds); break;
-        case 2: skinny_body<MODE, 2>(ga.x, w0, s0, w1, s1, y, m0, rows, n0, N, K, kbeg, kend, lds); break;
-        default: skinny_body<MODE, 3>(ga.x, w0, s0, w1, s1, y, m0, rows, n0, N, K, kbeg, kend, lds); break;
+        case 1: skinny_body<MODE, 1>(ga.x, w0, s0, w1, s1, y, rowidx, m0, rows, n0, N, K, kbeg, kend, lds); break;
+        case 2: skinny_body<MODE, 2>(ga.x, w0, s0, w1, s1, y, rowidx, m0, rows, n0, N, K, kbeg, kend, lds); break;
+        default: skinny_body<MODE, 3>(ga.x, w0, s0, w1, s1, y, rowidx, m0, rows, n0, N, K, kbeg, kend, lds); break;
     }
 }
 
 bool gemm_skinny_ok(int H, int F) { return H % 256 == 0 && F % 256 == 0; }
 
 template <int MODE>
-static int skinny_launch(const GemmGroup *groups, const int32_t *tiles, int mtiles, int E, int ntiles, int N, int K, int ksplit,
-                         size_t ystride, hipStream_t st) {
+static int skinny_launch(const GemmGroup *groups, const int32_t *tiles, const int32_t *tok, int mtiles, int E, int ntiles, int N,
+                         int K, int ksplit, size_t ystride, hipStream_t st) {
     static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
     if (!attr_set.load(std::memory_order_acquire)) {
         CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_skinny_i4g32_kernel<MODE>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS));
         attr_set.store(true, std::memory_order_release);
     }
-    hipLaunchKernelGGL((gemm_skinny_i4g32_kernel<MODE>), dim3(ntiles, mtiles, ksplit), dim3(256), SK_LDS, st, groups, tiles, E, N, K,
-                       K / ksplit, ystride);
+    hipLaunchKernelGGL((gemm_skinny_i4g32_kernel<MODE>), dim3(ntiles, mtiles, ksplit), dim3(256), SK_LDS, st, groups, tiles, tok, E, N,
+                       K, K / ksplit, ystride);
     return hip_check(hipGetLastError(), "gemm_skinny launch");
 }
 
 int gemm_skinny_tile_rows() { return SK_MT; }
 
-// gate/up with the SiLU epilogue: h[P,F] bf16 (through the down descriptors' x pointers)
-int gemm_skinny_gateup(const GemmGroup *groups, const int32_t *tiles, int ntiles, int E, int F, int H, hipStream_t st) {
-    return skinny_launch<1>(groups, tiles, ntiles, E, F / 128, F, H, 1, 0, st);
+// gate/up with the SiLU epilogue: h[P,F] bf16 (through the down descriptors' x pointers).  tok != nullptr: the
+// descriptors address the activations through the token of each row instead of a gathered copy.
+int gemm_skinny_gateup(const GemmGroup *groups, const int32_t *tiles, const int32_t *tok, int ntiles, int E, int F, int H,
+                       hipStream_t st) {
+    return skinny_launch<1>(groups, tiles, tok, ntiles, E, F / 128, F, H, 1, 0, st);
 }
 
 // down: fp32 parts [ksplit][P,H]
 int gemm_skinny_down(const GemmGroup *groups, const int32_t *tiles, int ntiles, int E, int H, int F, int ksplit, size_t ysplit_stride,
                      hipStream_t st) {
-    return skinny_launch<0>(groups, tiles, ntiles, E, H / 256, H, F, ksplit, ysplit_stride, st);
+    return skinny_launch<0>(groups, tiles, nullptr, ntiles, E, H / 256, H, F, ksplit, ysplit_stride, st);
 }
 
 }  // namespace chadq

@@ -4,10 +4,11 @@
 //
 // Everything runs on the caller's stream without a host round trip: the router kernel also sorts the
 // (token, slot) pairs by expert (stable: by pair index inside an expert) and writes the per-expert descriptors
-// of three grouped GEMM launches (gate, up: fp32 out; down: fp32 out), whose row counts therefore never
-// leave the GPU.  Gate/up/down run on the skinny grouped kernel (gate and up fused with the SiLU gate, down split
-// over K) when H and F are multiples of 256, else on the prefill dequant-GEMM kernel in grouped mode with a
-// separate SiLU kernel; the small kernels here are the gather, the SiLU gate and the weighted combine.
+// of the grouped GEMM launches and the list of token tiles that exist, so row counts never leave the GPU.
+// Gate/up/down run on the skinny grouped kernel (gate and up fused with the SiLU gate and reading the activations
+// through the sorted token list, down split over K) when H and F are multiples of 256, else on the prefill
+// dequant-GEMM kernel in grouped mode on a gathered copy of the activations with a separate SiLU kernel; the small
+// kernels here are the router, the gather, the SiLU gate and the weighted combine.
 #include "chadq_common.h"
 
 namespace chadq {
@@ -38,7 +39,8 @@ constexpr int MOE_KSPLIT = 4;
 int gemm_i4g32_grouped(const GemmGroup *groups, int ngroups, int m_max, int N, int K, bool out_f32, hipStream_t st);
 bool gemm_skinny_ok(int H, int F);
 int gemm_skinny_tile_rows();
-int gemm_skinny_gateup(const GemmGroup *groups, const int32_t *tiles, int ntiles, int E, int F, int H, hipStream_t st);
+int gemm_skinny_gateup(const GemmGroup *groups, const int32_t *tiles, const int32_t *tok, int ntiles, int E, int F, int H,
+                       hipStream_t st);
 int gemm_skinny_down(const GemmGroup *groups, const int32_t *tiles, int ntiles, int E, int H, int F, int ksplit, size_t ysplit_stride,
                      hipStream_t st);
 
@@ -46,10 +48,12 @@ int gemm_skinny_down(const GemmGroup *groups, const int32_t *tiles, int ntiles, 
 // Phase 3: descriptors.  idx/w may be the caller's arrays (chadq_moe_route) with everything else null.
 __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict__ logits, int32_t *__restrict__ idx,
                                                          float *__restrict__ w, int T, int E, int top_k, int renorm,
-                                                         MoeWs ws, MoeExperts ex, int H, int F) {
+                                                         MoeWs ws, MoeExperts ex, int H, int F,
+                                                         const uint16_t *__restrict__ x_src, int tile_rows, int ntiles_max) {
     __shared__ int s_base[MOE_MAX_E];   // rows of expert e seen so far
     __shared__ int s_cnt[16][MOE_MAX_E];  // per-wave counts of every expert in the current chunk
     __shared__ int s_off[MOE_MAX_E + 1];
+    __shared__ int s_tn[4 * MOE_MAX_E];  // token tiles per (fullness class, expert)
     // expert and rank of every pair stay in LDS between the phases when they fit (a global write followed by a read
     // from other threads costs a memory round trip per phase)
     constexpr int LP = 4096;
@@ -163,30 +167,46 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
     }
     if (tid < E) {
         const int e = tid, o = s_off[e], m = s_base[e];
-        ws.groups[e] = GemmGroup{ws.xs + (size_t)o * H, e_wg, e_sg, ws.g + (size_t)o * F, m, 0};
-        ws.groups[E + e] = GemmGroup{ws.xs + (size_t)o * H, e_wu, e_su, ws.u + (size_t)o * F, m, 0};
+        // x_src: the gate/up GEMM reads row tok[o + m] of the caller's activations; else rows o.. of the gathered copy
+        const uint16_t *xe = x_src ? x_src : ws.xs + (size_t)o * H;
+        ws.groups[e] = GemmGroup{xe, e_wg, e_sg, ws.g + (size_t)o * F, m, x_src ? o : 0};
+        ws.groups[E + e] = GemmGroup{xe, e_wu, e_su, ws.u + (size_t)o * F, m, x_src ? o : 0};
         ws.groups[2 * E + e] = GemmGroup{ws.h + (size_t)o * F, e_wd, e_sd, ws.yp + (size_t)o * H, m, 0};
+    }
+    // The token tiles of the expert GEMMs (expert | tile << 16, then -1), the fullest first: they take longest, and no
+    // workgroup is launched for a tile that does not exist except at the end of the grid.  Class c holds the tiles
+    // with tile_rows - 32c - 31 .. tile_rows - 32c rows; thread (c, e) counts expert e's tiles of class c, finds its
+    // place behind the classes and experts before it, and writes them.  Needs tile_rows <= 128.
+    if (ws.tiles && tile_rows > 0) {
+        const int ncls = (tile_rows + 31) >> 5;
+        int mine = 0, nfull = 0, cls_rem = -1;
+        if (tid < ncls * E) {
+            const int c = tid / E, m = s_base[tid % E];
+            nfull = m / tile_rows;
+            const int rem = m % tile_rows;
+            cls_rem = rem > 0 ? (tile_rows - rem) >> 5 : -1;
+            mine = (c == 0 ? nfull : 0) + (cls_rem == c ? 1 : 0);
+            s_tn[tid] = mine;
+        }
+        __syncthreads();
+        int total = 0;
+        for (int i = 0; i < ncls * E; ++i) total += s_tn[i];
+        if (tid < ncls * E) {
+            const int c = tid / E, e = tid % E;
+            int at = 0;
+            for (int i = 0; i < tid; ++i) at += s_tn[i];
+            if (c == 0)
+                for (int mt = 0; mt < nfull && at < ntiles_max; ++mt) ws.tiles[at++] = e | (mt << 16);
+            if (cls_rem == c && at < ntiles_max) ws.tiles[at] = e | (nfull << 16);
+        }
+        for (int n = total + tid; n < ntiles_max; n += B) ws.tiles[n] = -1;
     }
 }
 
-// xs[row] = x[tok[row]]; one 16-byte piece per thread.  Beside the copy, one thread of the last workgroup lists the
-// token tiles of the expert GEMMs (expert | tile << 16, then -1), the fullest first: they take longest, and no
-// workgroup is launched for a tile that does not exist except at the end of the grid.
+// xs[row] = x[tok[row]]; one 16-byte piece per thread.  Only the path through the prefill kernel needs the copy: the
+// skinny kernel reads the activations through tok.
 __global__ __launch_bounds__(256) void moe_gather_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ tok,
-                                                         uint16_t *__restrict__ xs, int P, int H, const int32_t *__restrict__ cnt,
-                                                         int32_t *__restrict__ tiles, int E, int tile_rows, int ntiles_max) {
-    if (tiles && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
-        int n = 0;
-        for (int lim = tile_rows; lim > 0 && n < ntiles_max; lim -= 32)  // classes of 32 rows: (lim - 32, lim]
-            for (int e = 0; e < E; ++e) {
-                const int m = cnt[e];
-                for (int mt = 0; mt * tile_rows < m; ++mt) {
-                    const int rows = min(m - mt * tile_rows, tile_rows);
-                    if (rows <= lim && rows > lim - 32 && n < ntiles_max) tiles[n++] = e | (mt << 16);
-                }
-            }
-        for (; n < ntiles_max; ++n) tiles[n] = -1;
-    }
+                                                         uint16_t *__restrict__ xs, int P, int H) {
     const int pieces = H / 8;
     const int64_t total = (int64_t)P * pieces, stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
@@ -263,7 +283,7 @@ size_t moe_workspace_bytes(int T, int H, int F, int E, int top_k) { return moe_l
 int moe_route_launch(const float *logits, int32_t *idx, float *w, int T, int E, int top_k, int renorm, hipStream_t st) {
     MoeWs ws = {};
     MoeExperts ex = {};
-    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 0, st, logits, idx, w, T, E, top_k, renorm, ws, ex, 0, 0);
+    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 0, st, logits, idx, w, T, E, top_k, renorm, ws, ex, 0, 0, nullptr, 0, 0);
     return hip_check(hipGetLastError(), "moe_route launch");
 }
 
@@ -283,17 +303,27 @@ int moe_ffn_i4g32_launch(const uint16_t *x, const float *logits, const chadq_moe
     const int P = T * top_k;
     const int m_max = P < T ? P : T;  // an expert gets a token at most once
     const int tile_rows = gemm_skinny_tile_rows(), ntiles = E + P / tile_rows;  // sum over experts of ceil(rows / tile_rows) <= this
-    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(P <= 256 ? 256 : P <= 512 ? 512 : 1024), 0, st, logits, ws.idx, ws.w, T, E, top_k, renorm, ws, ex, H, F);
-    hipLaunchKernelGGL(moe_gather_kernel, dim3(512), dim3(256), 0, st, x, ws.tok, ws.xs, P, H, ws.cnt, ws.tiles, E, tile_rows, ntiles);
-    int rc = hip_check(hipGetLastError(), "moe route/gather launch");
-    if (rc) return rc;
     int nsplit = 1;
     bool aligned = true;  // the skinny kernel loads scales 16 bytes at a time
     for (int e = 0; e < E; ++e)
         aligned = aligned && aligned16(experts[e].wg) && aligned16(experts[e].sg) && aligned16(experts[e].wu) &&
                   aligned16(experts[e].su) && aligned16(experts[e].wd) && aligned16(experts[e].sd);
-    if (aligned && gemm_skinny_ok(H, F)) {
-        rc = gemm_skinny_gateup(ws.groups, ws.tiles, ntiles, E, F, H, st);  // h = bf16(silu(gate) * up), [P,F]
+    const bool skinny = aligned && gemm_skinny_ok(H, F) && tile_rows <= 128;
+    const int route_threads = P <= 256 ? 256 : P <= 512 ? 512 : 1024;
+    int rc;
+    if (skinny) {  // the router also lists the token tiles; gate/up read the activations through tok
+        hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(route_threads), 0, st, logits, ws.idx, ws.w, T, E, top_k, renorm, ws, ex,
+                           H, F, x, tile_rows, ntiles);
+        rc = hip_check(hipGetLastError(), "moe route launch");
+    } else {
+        hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(route_threads), 0, st, logits, ws.idx, ws.w, T, E, top_k, renorm, ws, ex,
+                           H, F, nullptr, 0, 0);
+        hipLaunchKernelGGL(moe_gather_kernel, dim3(512), dim3(256), 0, st, x, ws.tok, ws.xs, P, H);
+        rc = hip_check(hipGetLastError(), "moe route/gather launch");
+    }
+    if (rc) return rc;
+    if (skinny) {
+        rc = gemm_skinny_gateup(ws.groups, ws.tiles, ws.tok, ntiles, E, F, H, st);  // h = bf16(silu(gate) * up), [P,F]
         if (rc) return rc;
         nsplit = (F % (256 * MOE_KSPLIT) == 0) ? MOE_KSPLIT : 1;
         rc = gemm_skinny_down(ws.groups, ws.tiles, ntiles, E, H, F, nsplit, (size_t)P * H, st);  // fp32 parts [nsplit][P,H]
