@@ -364,7 +364,10 @@ def test_moe_golden(ops):
 
 
 @pytest.mark.parametrize("t,h,f,e,top_k", [(256, 512, 1024, 8, 2), (37, 128, 160, 3, 1), (64, 256, 256, 1, 1), (130, 256, 512, 16, 4),
-                                           (300, 256, 512, 2, 2), (33, 256, 768, 8, 2), (200, 512, 512, 3, 1)])
+                                           (300, 256, 512, 2, 2), (33, 256, 768, 8, 2), (200, 512, 512, 3, 1),
+                                           # more than 1024 pairs (the router sorts them in several passes) and more than
+                                           # 4096 (its ranks go through memory instead of LDS)
+                                           (400, 256, 256, 8, 4), (1200, 256, 256, 4, 4), (1100, 64, 96, 5, 4)])
 def test_moe_ffn(ops, t, h, f, e, top_k):
     host, dev = _experts(80 + t, e, h, f)
     r = rng(81 + t)
