@@ -2,7 +2,7 @@
 //
 // HBM-bound stream of W.  A wavefront owns whole rows; one 128-bit load per lane = 16 weights, a wave-wide
 // load = 1024 consecutive k (1 KiB contiguous).  All loads of a wave are issued first; the fp32 activations
-// of the lane's k positions are read once and stay in registers.  Signed bytes are flipped to unsigned
+// come once per workgroup, through LDS, and a lane's k positions stay in registers.  Signed bytes are flipped to unsigned
 // (w ^ 0x80 = w + 128) so that v_cvt_f32_ubyteN converts them in one instruction; the accumulator starts
 // at -128 * sum(x) to take the offset back out.  DPP adds fold the 64 partial sums; no LDS.
 #include "chadq_common.h"
@@ -18,19 +18,20 @@ __global__ __launch_bounds__(256) void gemv_i8row_rows_kernel(const float *__res
                                                               int N, int K) {
     const int lane = threadIdx.x & 63;
     const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int row0 = gw * R;
-    if (row0 >= N) return;
+    const int row0 = gw * R;  // waves past the last row run on clamped rows and store nothing (no return before the barrier)
 
-    // activation loads first: memory returns in order, so waiting for them must not sit behind the weights
-    f32x4 xv[MB][CH][4];
+    // Activation loads first (memory returns in order, so waiting for them must not sit behind the weights): the
+    // workgroup fetches each activation once, CH 16-byte pieces per thread and row, and shares it through LDS -
+    // a quarter of the requests of every wave fetching its own copy.  Piece q (4 floats) lives at slot
+    // q ^ ((q >> 4) & 3), which makes the read-back below (lane l reads pieces 4l .. 4l+3) free of bank conflicts.
+    __shared__ __attribute__((aligned(16))) float sx[MB][CH * 1024];
+    f32x4 xg[MB][CH];
 #pragma unroll
     for (int m = 0; m < MB; ++m)
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
-            const int k0 = c * 1024 + lane * 16;
-            const f32x4 *xp = reinterpret_cast<const f32x4 *>(x + (size_t)m * K + ((k0 < K) ? k0 : 0));
-#pragma unroll
-            for (int i = 0; i < 4; ++i) xv[m][c][i] = xp[i];
+            const int k0 = (c * 256 + (int)threadIdx.x) * 4;
+            xg[m][c] = *reinterpret_cast<const f32x4 *>(x + (size_t)m * K + ((k0 < K) ? k0 : 0));
         }
 
     u32x4 w[R][CH];
@@ -46,6 +47,16 @@ __global__ __launch_bounds__(256) void gemv_i8row_rows_kernel(const float *__res
     }
     __builtin_amdgcn_sched_barrier(0);  // every load above is issued before anything below may wait
 
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int q = c * 256 + (int)threadIdx.x;
+            f32x4 v = xg[m][c];
+            if (q * 4 >= K) v = f32x4{0.f, 0.f, 0.f, 0.f};
+            *reinterpret_cast<f32x4 *>(&sx[m][(q ^ ((q >> 4) & 3)) * 4]) = v;
+        }
+    __syncthreads();
     float xs[MB][CH][16];
     float bias[MB];
 #pragma unroll
@@ -53,11 +64,10 @@ __global__ __launch_bounds__(256) void gemv_i8row_rows_kernel(const float *__res
         float sum = 0.f;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
-            const bool ok = (c * 1024 + lane * 16) < K;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                f32x4 v = xv[m][c][i];
-                if (!ok) v = f32x4{0.f, 0.f, 0.f, 0.f};
+                const int q = c * 256 + lane * 4 + i;
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(&sx[m][(q ^ ((q >> 4) & 3)) * 4]);
                 xs[m][c][4 * i + 0] = v.x;
                 xs[m][c][4 * i + 1] = v.y;
                 xs[m][c][4 * i + 2] = v.z;
