@@ -11,13 +11,13 @@ namespace chadq {
 
 __device__ __forceinline__ float ubyte_to_f32(uint32_t v, int i) { return (float)((v >> (8 * i)) & 0xFFu); }
 
-template <int CH, int R, int MB>
-__global__ __launch_bounds__(256) void gemv_i8row_rows_kernel(const float *__restrict__ x,
+template <int CH, int R, int MB, int WPB>
+__global__ __launch_bounds__(64 * WPB) void gemv_i8row_rows_kernel(const float *__restrict__ x,
                                                               const int8_t *__restrict__ w8,
                                                               const float *__restrict__ sc, float *__restrict__ y,
                                                               int N, int K) {
     const int lane = threadIdx.x & 63;
-    const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int gw = blockIdx.x * WPB + (threadIdx.x >> 6);
     const int row0 = gw * R;  // waves past the last row run on clamped rows and store nothing (no return before the barrier)
 
     // Activation loads first (memory returns in order, so waiting for them must not sit behind the weights): the
@@ -25,12 +25,13 @@ __global__ __launch_bounds__(256) void gemv_i8row_rows_kernel(const float *__res
     // a quarter of the requests of every wave fetching its own copy.  Piece q (4 floats) lives at slot
     // q ^ ((q >> 4) & 3), which makes the read-back below (lane l reads pieces 4l .. 4l+3) free of bank conflicts.
     __shared__ __attribute__((aligned(16))) float sx[MB][CH * 1024];
-    f32x4 xg[MB][CH];
+    constexpr int T = 64 * WPB, XP = (CH * 256 + T - 1) / T;  // threads, pieces per thread and row
+    f32x4 xg[MB][XP];
 #pragma unroll
     for (int m = 0; m < MB; ++m)
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int k0 = (c * 256 + (int)threadIdx.x) * 4;
+        for (int c = 0; c < XP; ++c) {
+            const int k0 = (c * T + (int)threadIdx.x) * 4;
             xg[m][c] = *reinterpret_cast<const f32x4 *>(x + (size_t)m * K + ((k0 < K) ? k0 : 0));
         }
 
@@ -50,11 +51,11 @@ __global__ __launch_bounds__(256) void gemv_i8row_rows_kernel(const float *__res
 #pragma unroll
     for (int m = 0; m < MB; ++m)
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int q = c * 256 + (int)threadIdx.x;
+        for (int c = 0; c < XP; ++c) {
+            const int q = c * T + (int)threadIdx.x;
             f32x4 v = xg[m][c];
             if (q * 4 >= K) v = f32x4{0.f, 0.f, 0.f, 0.f};
-            *reinterpret_cast<f32x4 *>(&sx[m][(q ^ ((q >> 4) & 3)) * 4]) = v;
+            if (q < CH * 256) *reinterpret_cast<f32x4 *>(&sx[m][(q ^ ((q >> 4) & 3)) * 4]) = v;
         }
     __syncthreads();
     float xs[MB][CH][16];
@@ -135,14 +136,17 @@ __global__ __launch_bounds__(256) void gemv_i8row_generic_kernel(const float *__
     }
 }
 
-template <int CH, int R, int MB>
+template <int CH, int R, int MB, int WPB>
 static void launch_rows8(const float *x, const int8_t *w8, const float *sc, float *y, int N, int K, hipStream_t st) {
     const int waves = (N + R - 1) / R;
-    hipLaunchKernelGGL((gemv_i8row_rows_kernel<CH, R, MB>), dim3((waves + 3) / 4), dim3(256), 0, st, x, w8, sc, y, N, K);
+    hipLaunchKernelGGL((gemv_i8row_rows_kernel<CH, R, MB, WPB>), dim3((waves + WPB - 1) / WPB), dim3(64 * WPB), 0, st, x, w8, sc, y,
+                       N, K);
 }
 
 int gemv_i8row_dispatch(const float *x, const int8_t *w8, const float *sc, float *y, int M, int N, int K,
                         hipStream_t st) {
+    // <1024-wide chunks per row, rows per wave, activation rows, waves per workgroup>, picked by measurement: eight
+    // waves share one copy of the activations; matrices with many rows give a wave 2 or 4 rows
     if (K <= 2048) {
         const bool big = N >= 8192;
         for (int m0 = 0; m0 < M;) {
@@ -150,11 +154,11 @@ int gemv_i8row_dispatch(const float *x, const int8_t *w8, const float *sc, float
             float *ym = y + (size_t)m0 * N;
             const int mb = (M - m0 >= 2) ? 2 : 1;
             if (K <= 1024) {
-                if (mb == 2) big ? launch_rows8<1, 8, 2>(xm, w8, sc, ym, N, K, st) : launch_rows8<1, 2, 2>(xm, w8, sc, ym, N, K, st);
-                else big ? launch_rows8<1, 8, 1>(xm, w8, sc, ym, N, K, st) : launch_rows8<1, 2, 1>(xm, w8, sc, ym, N, K, st);
+                if (mb == 2) big ? launch_rows8<1, 4, 2, 8>(xm, w8, sc, ym, N, K, st) : launch_rows8<1, 2, 2, 8>(xm, w8, sc, ym, N, K, st);
+                else big ? launch_rows8<1, 4, 1, 8>(xm, w8, sc, ym, N, K, st) : launch_rows8<1, 2, 1, 8>(xm, w8, sc, ym, N, K, st);
             } else {
-                if (mb == 2) big ? launch_rows8<2, 4, 2>(xm, w8, sc, ym, N, K, st) : launch_rows8<2, 1, 2>(xm, w8, sc, ym, N, K, st);
-                else big ? launch_rows8<2, 4, 1>(xm, w8, sc, ym, N, K, st) : launch_rows8<2, 1, 1>(xm, w8, sc, ym, N, K, st);
+                if (mb == 2) big ? launch_rows8<2, 2, 2, 8>(xm, w8, sc, ym, N, K, st) : launch_rows8<2, 1, 2, 8>(xm, w8, sc, ym, N, K, st);
+                else big ? launch_rows8<2, 2, 1, 8>(xm, w8, sc, ym, N, K, st) : launch_rows8<2, 1, 1, 8>(xm, w8, sc, ym, N, K, st);
             }
             m0 += mb;
         }
