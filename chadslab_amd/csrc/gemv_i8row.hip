@@ -162,6 +162,13 @@ int gemv_i8row_dispatch(const float *x, const int8_t *w8, const float *sc, float
             }
             m0 += mb;
         }
+    } else if (K <= 8192) {  // rows of up to 4096 / 8192 k: the same kernel with 4 or 8 chunks per row, one activation row at a time
+        for (int m0 = 0; m0 < M; ++m0) {
+            const float *xm = x + (size_t)m0 * K;
+            float *ym = y + (size_t)m0 * N;
+            if (K <= 4096) N >= 4096 ? launch_rows8<4, 2, 1, 8>(xm, w8, sc, ym, N, K, st) : launch_rows8<4, 1, 1, 8>(xm, w8, sc, ym, N, K, st);
+            else launch_rows8<8, 1, 1, 8>(xm, w8, sc, ym, N, K, st);
+        }
     } else {
         hipLaunchKernelGGL(gemv_i8row_generic_kernel, dim3((N + 3) / 4), dim3(256), 0, st, x, w8, sc, y, M, N, K);
     }

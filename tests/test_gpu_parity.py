@@ -201,7 +201,10 @@ def test_gemv_int4_zero_weights_and_special_scales(ops):
 
 
 # ------------------------------------------------------------------ GEMV int8 (config 0)
-@pytest.mark.parametrize("m,n,k", [(1, 16384, 2048), (1, 64, 16), (3, 100, 1040), (2, 77, 4096), (16, 40, 256)])
+@pytest.mark.parametrize("m,n,k", [(1, 16384, 2048), (1, 64, 16), (3, 100, 1040), (2, 77, 4096), (16, 40, 256),
+                                   # rows of 2049..8192 k (4 or 8 chunks per row), and beyond (the general kernel)
+                                   (1, 5000, 4096), (2, 300, 3008), (1, 4500, 8192), (3, 33, 6000), (1, 50, 8208),
+                                   (1, 9000, 1024), (2, 8200, 528)])
 def test_gemv_int8(ops, m, n, k):
     x, w, s, q8 = i8_case(1000 if (n, k) == (16384, 2048) else 20 + n, m, n, k)
     y = ops.qgemv(torch.from_numpy(x).to(DEV), q8).cpu().numpy()
