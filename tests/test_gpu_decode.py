@@ -335,6 +335,28 @@ def test_sample_topk_matches_the_oracle(lib, n, k, temperature):
     assert checked >= 25 and int(pos.item()) == 7 + 32
 
 
+@pytest.mark.parametrize("n,k,levels", [(256000, 50, 6), (256000, 64, 3), (5000, 20, 2), (700, 64, 40), (256000, 7, 5), (300, 64, 1)])
+def test_sample_topk_with_many_equal_logits(lib, n, k, levels):
+    # few distinct values: the k-th best lies inside a run of equal logits, of which the lowest indices are candidates
+    r = rng(2000 + n + k)
+    v = (r.integers(0, levels, n) * 0.25).astype(np.float32)
+    v[r.integers(0, n, 5)] = np.nan
+    v[r.integers(0, n, 3)] = -np.inf
+    v[n // 2] = -0.0 if levels == 1 else v[n // 2]
+    t = dev(v)
+    ws = torch.zeros(49152 // 4, dtype=torch.float32, device=DEV)
+    tok = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    checked = 0
+    for u in np.concatenate([[0.0, 0.999999], r.random(40)]).astype(np.float32):
+        ud = torch.tensor([u], dtype=torch.float32, device=DEV)
+        chk(lib.chadq_sample_topk_f32(t.data_ptr(), n, k, 1.0, ud.data_ptr(), ws.data_ptr(), tok.data_ptr(), None, 0, stream()),
+            "sample_topk")
+        if _sample_margin(v, k, 1.0, float(u)) > 1e-5:
+            assert int(tok.item()) == O.sample_topk(v, k, 1.0, float(u)), (n, k, levels, u)
+            checked += 1
+    assert checked >= 30
+
+
 def test_sample_topk_rejects_bad_arguments(lib):
     t = dev(np.zeros(100, np.float32))
     ws = torch.zeros(49152 // 4, dtype=torch.float32, device=DEV)
