@@ -8,6 +8,8 @@
 //   FFN: GeGLU with the tanh form of GELU.   Embedding: the tied int4 output table, dequantised row.
 #include <type_traits>
 
+#include <climits>
+
 #include "chadq_common.h"
 
 namespace chadq {
@@ -550,67 +552,76 @@ __global__ __launch_bounds__(256) void geglu_kernel(const float *__restrict__ gu
     }
 }
 
-// argmax over n fp32 values (lowest index wins ties): per-workgroup candidates, then one workgroup; the winner
-// becomes the next token and the position advances, so that a replayed graph steps by itself.
-__global__ __launch_bounds__(256) void argmax_partial_kernel(const float *__restrict__ v, int n, float *__restrict__ pv,
-                                                             int32_t *__restrict__ pi) {
-    __shared__ float sv[256];
-    __shared__ int si[256];
-    float best = -INFINITY;
-    int bi = 0x7fffffff;
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
-        if (v[i] > best || (v[i] == best && i < bi)) {
-            best = v[i];
-            bi = i;
+// argmax over n fp32 values (lowest index wins ties, NaN is never the winner; token 0 if every value is NaN):
+// per-workgroup candidates, then one workgroup; the winner becomes the next token and the position advances, so that
+// a replayed graph steps by itself.  A thread keeps the best of its elements (loads four at a time), a wave finds its
+// winner with DPP moves and a ballot, and the four waves meet once in LDS.
+__device__ __forceinline__ void argmax_block(float best, int bi, float *out_v, int32_t *out_i) {
+    __shared__ float s_v[4];
+    __shared__ int32_t s_i[4];
+    const int wave = threadIdx.x >> 6;
+    const uint32_t gi = wave_winner<64>(bi != INT_MAX, best, bi);
+    if (gi == 0xFFFFFFFFu) {
+        if ((threadIdx.x & 63) == 0) {
+            s_v[wave] = -INFINITY;
+            s_i[wave] = INT_MAX;
         }
-    sv[threadIdx.x] = best;
-    si[threadIdx.x] = bi;
-    __syncthreads();
-    for (int o = 128; o > 0; o >>= 1) {
-        if ((int)threadIdx.x < o) {
-            const float ov = sv[threadIdx.x + o];
-            const int oi = si[threadIdx.x + o];
-            if (ov > sv[threadIdx.x] || (ov == sv[threadIdx.x] && oi < si[threadIdx.x])) {
-                sv[threadIdx.x] = ov;
-                si[threadIdx.x] = oi;
-            }
-        }
-        __syncthreads();
+    } else if ((uint32_t)bi == gi) {  // one lane: indices are distinct
+        s_v[wave] = best;
+        s_i[wave] = bi;
     }
+    __syncthreads();
     if (threadIdx.x == 0) {
-        pv[blockIdx.x] = sv[0];
-        pi[blockIdx.x] = si[0];
+        float bv = s_v[0];
+        int bb = s_i[0];
+#pragma unroll
+        for (int w = 1; w < 4; ++w)
+            if (s_i[w] != INT_MAX && (bb == INT_MAX || s_v[w] > bv || (s_v[w] == bv && s_i[w] < bb))) {
+                bv = s_v[w];
+                bb = s_i[w];
+            }
+        *out_v = bv;
+        *out_i = bb;
     }
 }
 
-__global__ __launch_bounds__(256) void argmax_final_kernel(const float *__restrict__ pv, const int32_t *__restrict__ pi, int nb,
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float *__restrict__ v, int n, float *__restrict__ pv,
+                                                             int32_t *__restrict__ pi) {
+    float best = -INFINITY;
+    int bi = INT_MAX;
+    const int stride = gridDim.x * blockDim.x;
+    for (int i0 = blockIdx.x * blockDim.x + threadIdx.x; i0 < n; i0 += 4 * stride) {
+        float x[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) x[j] = (i0 + j * stride < n) ? v[i0 + j * stride] : __builtin_nanf("");
+#pragma unroll
+        for (int j = 0; j < 4; ++j)  // increasing index: an equal value later never replaces an earlier one
+            if (x[j] > best || (x[j] == best && bi == INT_MAX)) {
+                best = x[j];
+                bi = i0 + j * stride;
+            }
+    }
+    argmax_block(best, bi, pv + blockIdx.x, pi + blockIdx.x);
+}
+
+__global__ __launch_bounds__(256) void argmax_final_kernel(const float *__restrict__ pv, const int32_t *__restrict__ pi, int nb, int n,
                                                            int32_t *__restrict__ token, int32_t *__restrict__ pos,
                                                            int advance) {
-    __shared__ float sv[256];
-    __shared__ int si[256];
+    __shared__ float fv;
+    __shared__ int32_t fi;
     float best = -INFINITY;
-    int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < nb; i += blockDim.x)
-        if (pv[i] > best || (pv[i] == best && pi[i] < bi)) {
-            best = pv[i];
-            bi = pi[i];
+    int bi = INT_MAX;
+    for (int i = threadIdx.x; i < nb; i += blockDim.x) {
+        const float x = pv[i];
+        const int xi = pi[i];
+        if (xi != INT_MAX && (bi == INT_MAX || x > best || (x == best && xi < bi))) {
+            best = x;
+            bi = xi;
         }
-    sv[threadIdx.x] = best;
-    si[threadIdx.x] = bi;
-    __syncthreads();
-    for (int o = 128; o > 0; o >>= 1) {
-        if ((int)threadIdx.x < o) {
-            const float ov = sv[threadIdx.x + o];
-            const int oi = si[threadIdx.x + o];
-            if (ov > sv[threadIdx.x] || (ov == sv[threadIdx.x] && oi < si[threadIdx.x])) {
-                sv[threadIdx.x] = ov;
-                si[threadIdx.x] = oi;
-            }
-        }
-        __syncthreads();
     }
+    argmax_block(best, bi, &fv, &fi);
     if (threadIdx.x == 0) {
-        token[0] = si[0];
+        token[0] = (fi == INT_MAX) ? 0 : min(max(fi, 0), n - 1);
         if (advance) pos[0] += 1;
     }
 }
@@ -681,7 +692,7 @@ int geglu_launch(const float *gu, uint16_t *h, int F, hipStream_t st) {
 int argmax_launch(const float *v, int n, float *pv, int32_t *pi, int32_t *token, int32_t *pos, int advance, hipStream_t st) {
     const int nb = 256;
     hipLaunchKernelGGL(argmax_partial_kernel, dim3(nb), dim3(256), 0, st, v, n, pv, pi);
-    hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, st, pv, pi, nb, token, pos, advance);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, st, pv, pi, nb, n, token, pos, advance);
     return hip_check(hipGetLastError(), "argmax launch");
 }
 

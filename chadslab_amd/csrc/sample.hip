@@ -19,48 +19,6 @@ namespace chadq {
 constexpr int TOPK_MAX = 64, TOPK_NB = 96;  // a lane holds up to 32 logits: the entry point limits n to 96 * 4 * 64 * 32
 constexpr int TOPK_PICK_MIN = 16;           // k from which the selection by threshold is used (the rounds cost 5 + 1.25 k us, it 23-29)
 
-// floats as unsigned keys of the same order; -0 and +0 get the same key
-__device__ __forceinline__ uint32_t order_key(float v) {
-    const uint32_t b = __float_as_uint(v + 0.f);
-    return b ^ ((b >> 31) ? 0xFFFFFFFFu : 0x80000000u);
-}
-
-// max (or min) of an unsigned value over the first LANES lanes of the wave (64, or 4: one quad), returned to every lane:
-// butterflies inside the 16-lane rows, then the two row broadcasts gather the total in lane 63.  Lanes a DPP move
-// does not reach receive the operation's identity, so that the compiler can fold each move into its max / min.
-template <bool IS_MAX, int LANES>
-__device__ __forceinline__ uint32_t wave_reduce_u32(uint32_t v) {
-    constexpr int IDENT = IS_MAX ? 0 : -1;
-#define CHADQ_DPP_STEP(CTRL, MASK)                                                                                  \
-    {                                                                                                               \
-        const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(IDENT, (int)v, CTRL, MASK, 0xF, false);            \
-        v = IS_MAX ? (o > v ? o : v) : (o < v ? o : v);                                                             \
-    }
-    CHADQ_DPP_STEP(0xB1, 0xF)  // quad_perm [1,0,3,2]
-    CHADQ_DPP_STEP(0x4E, 0xF)  // quad_perm [2,3,0,1]
-    if (LANES == 4) return (uint32_t)__builtin_amdgcn_readlane((int)v, 0);
-    CHADQ_DPP_STEP(0x141, 0xF)  // row_half_mirror
-    CHADQ_DPP_STEP(0x140, 0xF)  // row_mirror
-    CHADQ_DPP_STEP(0x142, 0xA)  // row_bcast15 into rows 1 and 3
-    CHADQ_DPP_STEP(0x143, 0xC)  // row_bcast31 into rows 2 and 3
-#undef CHADQ_DPP_STEP
-    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
-}
-
-// The winner among one (value, index) pair per lane (has = false: the lane has none): the largest value, the lowest
-// index among equal values.  Returns the winner's index, or 0xFFFFFFFF if no lane has a pair.  One reduction finds the
-// largest value; a second one, over the indices, runs only when several lanes hold it.
-template <int LANES>
-__device__ __forceinline__ uint32_t wave_winner(bool has, float v, int i) {
-    const uint32_t key = has ? order_key(v) : 0u;  // below the key of -inf
-    const uint32_t best = wave_reduce_u32<true, LANES>(key);
-    const bool match = has && key == best;
-    const unsigned long long m = __ballot(match);
-    if (m == 0) return 0xFFFFFFFFu;
-    if ((m & (m - 1)) == 0) return (uint32_t)__builtin_amdgcn_readlane(i, __ffsll((long long)m) - 1);
-    return wave_reduce_u32<false, LANES>(match ? (uint32_t)i : 0xFFFFFFFFu);
-}
-
 // One wave moves the k first of the `cnt` values v[base ..] to ov/oi, in order.  Lane holds elements lane + 64 j, j < E,
 // in registers (cnt <= 64 E); a taken or absent element is NaN, which is never a candidate.  Missing places are
 // filled with (-inf, INT_MAX).
