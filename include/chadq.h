@@ -209,7 +209,8 @@ int chadq_attn_decode_mqa_fused(const float *qkv, const int32_t *pos, const floa
 int chadq_geglu_bf16(const float *gu, uint16_t *h_bf16, int F, void *stream);
 
 /*
- * token[0] = argmax of v[0..n) (lowest index wins ties); pos[0] += 1 if advance != 0.
+ * token[0] = argmax of v[0..n) (lowest index wins ties; NaN never wins; 0 if every value is NaN); pos[0] += 1 if
+ * advance != 0.
  * scratch: 256 floats followed by 256 int32 (2048 bytes).
  */
 int chadq_argmax_f32(const float *v, int n, void *scratch, int32_t *token, int32_t *pos, int advance, void *stream);
