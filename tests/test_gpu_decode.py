@@ -310,6 +310,33 @@ def _sample_margin(v, k, temperature, u):
     return float(np.abs(c / c[-1] - u).min())
 
 
+@pytest.mark.parametrize("n", [5, 300, 256000, 1500000])
+def test_argmax_special_values(lib, n):
+    # NaN never wins; among equal values (-inf, -0/+0, runs of the maximum) the lowest index; all NaN gives token 0
+    r = rng(50 + n)
+    scratch = torch.zeros(512, dtype=torch.float32, device=DEV)
+    tok = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+
+    def run(v):
+        chk(lib.chadq_argmax_f32(dev(v).data_ptr(), n, scratch.data_ptr(), tok.data_ptr(), None, 0, stream()), "argmax")
+        return int(tok.item())
+
+    v = r.standard_normal(n).astype(np.float32)
+    v[r.integers(0, n, max(1, n // 7))] = np.nan
+    assert run(v) == int(np.nanargmax(v))
+    v = np.full(n, -np.inf, np.float32)
+    v[0] = np.nan
+    assert run(v) == (1 if n > 1 else 0)
+    v = np.full(n, np.nan, np.float32)
+    assert run(v) == 0
+    v = np.zeros(n, np.float32)
+    v[n // 2:] = -0.0
+    v[0] = -1.0
+    assert run(v) == 1
+    v = (r.integers(0, 3, n)).astype(np.float32)  # long runs of the maximum
+    assert run(v) == int(np.argmax(v))
+
+
 @pytest.mark.parametrize("n,k,temperature", [(256000, 1, 1.0), (256000, 8, 0.7), (256000, 50, 1.0), (256000, 64, 1.3),
                                              (1000, 64, 1.0), (97, 5, 0.5), (5, 5, 1.0), (1, 1, 1.0), (786432, 40, 1.0)])
 def test_sample_topk_matches_the_oracle(lib, n, k, temperature):
