@@ -267,21 +267,41 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
 // (expert | tile << 16, -1 past the last), also from the router, fullest first.  MODE 1 with tok != nullptr: the
 // gate/up descriptors' x is the ungathered activation matrix and `pad` the expert's first row in tok, the token of
 // every expert-sorted row.
-// grid: x = N tiles, y = entry of the tile list, z = K split (MODE 0 only).
+// grid: one dimension, decoded in the kernel into n-tile, entry of the tile list and K split (MODE 0 only).
 template <int MODE>
 __global__ __launch_bounds__(256, SK_WGS_PER_CU) void gemm_skinny_i4g32_kernel(const GemmGroup *__restrict__ groups,
                                                                   const int32_t *__restrict__ tiles,
                                                                   const int32_t *__restrict__ tok, int E, int N, int K,
-                                                                  int kspan, size_t ysplit_stride) {
+                                                                  int kspan, size_t ysplit_stride, int nx, int ny, int nz) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const int tile = tiles[blockIdx.y];
+    // Workgroup -> (n-tile bx, list entry by, K split bz).  Workgroup i runs on XCD i % 8, each with its own L2.
+    // Down projection: the nx n-tiles of one (entry, split) read the same activation rows, so they are dealt to ONE XCD
+    // (spread over all of them, every XCD fetched the routed activations once: a quarter of the kernel's memory
+    // traffic); pairs count splits fastest, so the entries that exist (the first of the list) come out evenly.
+    // Gate/up: n-tiles fastest, which spreads every expert over all XCDs whatever the experts' sizes (its activation
+    // tiles fit the L2s anyway).
+    int bx, by, bz;
+    if (MODE == 1) {
+        bx = blockIdx.x % nx;
+        by = blockIdx.x / nx;
+        bz = 0;
+        if (by >= ny) return;
+    } else {
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        const int pair = (slot / nx) * 8 + xcd;
+        bx = slot % nx;
+        if (pair >= ny * nz) return;
+        by = pair / nz;
+        bz = pair % nz;
+    }
+    const int tile = tiles[by];
     if (tile < 0) return;
     const int g = tile & 0xFFFF, mt = tile >> 16;
     const GemmGroup ga = groups[MODE == 1 ? g : 2 * E + g];
     const int M = ga.M, m0 = mt * SK_MT;
     if (m0 >= M) return;
     const int rows = (M - m0) < SK_MT ? (M - m0) : SK_MT;
-    const int kbeg = blockIdx.z * kspan, kend = (kbeg + kspan < K) ? kbeg + kspan : K;
+    const int kbeg = bz * kspan, kend = (kbeg + kspan < K) ? kbeg + kspan : K;
     const uint8_t *w0 = reinterpret_cast<const uint8_t *>(ga.w), *w1 = nullptr;
     const uint16_t *s0 = reinterpret_cast<const uint16_t *>(ga.sc), *s1 = nullptr;
     void *y;
@@ -291,10 +311,10 @@ __global__ __launch_bounds__(256, SK_WGS_PER_CU) void gemm_skinny_i4g32_kernel(c
         w1 = reinterpret_cast<const uint8_t *>(gu.w);
         s1 = reinterpret_cast<const uint16_t *>(gu.sc);
         y = const_cast<uint16_t *>(gd.x);  // the down projection's input rows of this expert
-        n0 = blockIdx.x * 128;
+        n0 = bx * 128;
     } else {
-        y = reinterpret_cast<float *>(ga.y) + (size_t)blockIdx.z * ysplit_stride;
-        n0 = blockIdx.x * 256;
+        y = reinterpret_cast<float *>(ga.y) + (size_t)bz * ysplit_stride;
+        n0 = bx * 256;
     }
     const int32_t *rowidx = (MODE == 1 && tok) ? tok + ga.pad : nullptr;
     switch ((rows + 31) >> 5) {
@@ -315,8 +335,9 @@ static int skinny_launch(const GemmGroup *groups, const int32_t *tiles, const in
                                       hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS));
         attr_set.store(true, std::memory_order_release);
     }
-    hipLaunchKernelGGL((gemm_skinny_i4g32_kernel<MODE>), dim3(ntiles, mtiles, ksplit), dim3(256), SK_LDS, st, groups, tiles, tok, E, N,
-                       K, K / ksplit, ystride);
+    const int pairs8 = (mtiles * ksplit + 7) / 8 * 8;  // (list entry, split) pairs, dealt to the 8 XCDs
+    hipLaunchKernelGGL((gemm_skinny_i4g32_kernel<MODE>), dim3(pairs8 * ntiles), dim3(256), SK_LDS, st, groups, tiles, tok, E, N, K,
+                       K / ksplit, ystride, ntiles, mtiles, ksplit);
     return hip_check(hipGetLastError(), "gemm_skinny launch");
 }
 
