@@ -296,6 +296,27 @@ def main():
                                          "bytes_per_token": wbytes + kvbytes, "GBps": round((wbytes + kvbytes) / us4 * 1e-3, 1),
                                          "frac_hbm_peak": round((wbytes + kvbytes) / us4 * 1e-3 / HBM_PEAK_GBS, 4),
                                          "context": "2048..2111", "launch": "one HIP graph per token"}
+        del dec
+        # the same step ending in a draw from the 50 most likely tokens instead of the argmax (the uniform number stays
+        # fixed during the replays: the draw's cost does not depend on it)
+        with torch.cuda.stream(stream):
+            dec = QuantDecoder(cfg4, w4, dev)
+            for li in range(cfg4.n_layers):
+                dec.kcache[li].normal_()
+                dec.vcache[li].normal_()
+            dec.token.fill_(5)
+            dec.pos.fill_(2040)
+            dec.set_sampling(50, 1.0, 1004)
+            dec.capture()
+            for _ in range(8):
+                dec.graph.replay()
+            a4, b4 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a4.record(stream)
+            for _ in range(n_dec):
+                dec.graph.replay()
+            b4.record(stream)
+            torch.cuda.synchronize()
+        extras["decode_step_config4"]["us_per_token_sampling_top50"] = round(a4.elapsed_time(b4) * 1000.0 / n_dec, 1)
         del dec, w4
         torch.cuda.empty_cache()
 
