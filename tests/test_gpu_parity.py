@@ -291,6 +291,44 @@ def test_gemm_int4_integer_exact_when_scales_are_one(ops):
     assert np.array_equal(bits(ops.qgemm(bf16_tensor(xb), ones)), O.f32_to_bf16(brute))
 
 
+# ------------------------------------------------------------------ full benchmark sizes: properties that need no CPU reference
+def test_full_size_properties_without_a_reference(ops):
+    from chadslab_amd import QWeightInt4G32, QWeightInt8
+
+    # config 1: rows of an M=8 product equal the M=1 products; integer inputs make linearity exact
+    n, k = 14336, 4096
+    packed, s, xb, qw = i4_case(1001, 8, n, k)
+    x = bf16_tensor(xb)
+    y8 = ops.qgemv(x, qw).cpu().numpy()
+    for r in (0, 5):
+        assert O.rel_l2(ops.qgemv(x[r:r + 1].contiguous(), qw).cpu().numpy()[0], y8[r]) <= 1e-6
+    ones = QWeightInt4G32(qw.packed, torch.ones_like(qw.scale))
+    a = rng(2).integers(-4, 5, (1, k)).astype(np.float32)
+    b = rng(3).integers(-4, 5, (1, k)).astype(np.float32)
+    ya, yb, yab = (ops.qgemv(bf16_tensor(O.f32_to_bf16(v)), ones).cpu().numpy() for v in (a, b, a + b))
+    assert np.array_equal(yab, ya + yb)
+    # config 2: the prefill kernel and the decode kernel agree on the rows they share
+    packed2, s2, xb2, qw2 = i4_case(1002, 512, 4096, 4096)
+    x2 = bf16_tensor(xb2)
+    gemm = O.bf16_to_f32(bits(ops.qgemm(x2, qw2)))
+    gemv = ops.qgemv(x2[100:108].contiguous(), qw2).cpu().numpy()
+    assert O.rel_l2(gemm[100:108], gemv) <= TOL_BF16
+    # ... and a permutation of the activation rows permutes the output rows, bit for bit
+    perm = rng(4).permutation(512)
+    gemm_p = bits(ops.qgemm(bf16_tensor(xb2[perm]), qw2))
+    assert np.array_equal(gemm_p, bits(ops.qgemm(x2, qw2))[perm])
+    # config 0: scaling a row's scale scales that output; integer inputs make linearity exact
+    x0, w0, s0, q8 = i8_case(1000, 1, 16384, 2048)
+    y0 = ops.qgemv(torch.from_numpy(x0).to(DEV), q8).cpu().numpy()
+    q8b = QWeightInt8(q8.w, q8.scale * 2.0)
+    assert np.array_equal(ops.qgemv(torch.from_numpy(x0).to(DEV), q8b).cpu().numpy(), 2.0 * y0)
+    q1 = QWeightInt8(q8.w, torch.ones_like(q8.scale))
+    ia = rng(5).integers(-8, 9, (1, 2048)).astype(np.float32)
+    ib = rng(6).integers(-8, 9, (1, 2048)).astype(np.float32)
+    za, zb, zab = (ops.qgemv(torch.from_numpy(v).to(DEV), q1).cpu().numpy() for v in (ia, ib, ia + ib))
+    assert np.array_equal(zab, za + zb)
+
+
 # ------------------------------------------------------------------ operator layer and error behaviour
 def test_qlinear_dispatch(ops):
     packed, s, xb, qw = i4_case(60, 6, 128, 256)
