@@ -69,6 +69,9 @@ int geglu_launch(const float *, uint16_t *, int, hipStream_t);
 int rope_table_launch(float *, int, int, float, hipStream_t);
 int attn_mqa_fused_launch(const float *, const int32_t *, const float *, uint16_t *, uint16_t *, float *, uint16_t *, int, int, int,
                           hipStream_t);
+int attn_mqa_fused_static_launch(const float *, const int32_t *, const float *, uint16_t *, uint16_t *, uint16_t *, int, int, int,
+                                 hipStream_t);
+int attn_mqa_fused_static_max_ctx();
 int argmax_launch(const float *, int, float *, int32_t *, int32_t *, int32_t *, int, hipStream_t);
 int probe_read_launch(const uint8_t *, size_t, uint32_t *, hipStream_t);
 int sample_topk_launch(const float *, int, int, float, const float *, float *, int32_t *, int32_t *, int32_t *, int, hipStream_t);
@@ -317,6 +320,21 @@ int chadq_attn_decode_mqa_fused(const float *qkv, const int32_t *pos, const floa
     CHADQ_REQUIRE(aligned16(qkv) && aligned16(rope_table) && aligned16(kcache_bf16), CHADQ_ERR_ALIGN,
                   "chadq_attn_decode_mqa_fused: qkv, rope_table and kcache must be 16-byte aligned");
     return attn_mqa_fused_launch(qkv, pos, rope_table, kcache_bf16, vcache_bf16, workspace, out_bf16, hq, dh, max_ctx, st);
+}
+
+int chadq_attn_decode_mqa_fused_static(const float *qkv, const int32_t *pos, const float *rope_table, uint16_t *kcache_bf16,
+                                       uint16_t *vcache_bf16, uint16_t *out_bf16, int hq, int dh, int max_ctx, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(hq >= 1 && hq <= 8 && dh >= 16 && dh <= 256 && dh % 16 == 0 && max_ctx >= 1, CHADQ_ERR_SHAPE,
+                  "chadq_attn_decode_mqa_fused_static: hq=%d dh=%d max_ctx=%d (hq <= 8, dh <= 256 and a multiple of 16)", hq, dh, max_ctx);
+    CHADQ_REQUIRE(max_ctx <= attn_mqa_fused_static_max_ctx(), CHADQ_ERR_WORKSPACE,
+                  "chadq_attn_decode_mqa_fused_static: max_ctx=%d exceeds the %d rows the built-in scratch covers "
+                  "(use chadq_attn_decode_mqa_fused with a workspace)", max_ctx, attn_mqa_fused_static_max_ctx());
+    CHADQ_REQUIRE(qkv && pos && rope_table && kcache_bf16 && vcache_bf16 && out_bf16, CHADQ_ERR_NULL,
+                  "chadq_attn_decode_mqa_fused_static: null pointer");
+    CHADQ_REQUIRE(aligned16(qkv) && aligned16(rope_table) && aligned16(kcache_bf16), CHADQ_ERR_ALIGN,
+                  "chadq_attn_decode_mqa_fused_static: qkv, rope_table and kcache must be 16-byte aligned");
+    return attn_mqa_fused_static_launch(qkv, pos, rope_table, kcache_bf16, vcache_bf16, out_bf16, hq, dh, max_ctx, st);
 }
 
 int chadq_geglu_bf16(const float *gu, uint16_t *h_bf16, int F, void *stream) {
