@@ -9,7 +9,7 @@ embedding / output table without embedding scaling or logit soft-capping.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List
+from typing import Dict, List, Optional
 
 import torch
 
@@ -130,8 +130,11 @@ class QuantDecoder:
                                                    w.data_ptr(), self.xn.data_ptr(), self.cfg.d, self.cfg.eps, self._s()),
                    "chadq_add_rmsnorm_bf16")
 
-    def step(self) -> None:
-        """One token: reads token/pos from device memory, leaves the next token and pos+1 there."""
+    def step(self, trace: Optional[list] = None) -> None:
+        """One token: reads token/pos from device memory, leaves the next token and pos+1 there.  The caller keeps
+        pos below max_ctx (feed() and generate() check it on the host; the kernels only clamp for memory safety).
+        trace (eager launches only, for parity checks): receives a copy of the fp32 residual vector entering every
+        layer, then of the one entering the final norm (n_layers + 1 tensors)."""
         c, lib, s = self.cfg, self.lib, self._s()
         _lib.check(lib.chadq_embed_i4g32(self.token.data_ptr(), self.w["emb"].packed.data_ptr(), self.w["emb"].scale.data_ptr(),
                                          self.x.data_ptr(), c.d, c.vocab, s), "chadq_embed_i4g32")
@@ -147,6 +150,8 @@ class QuantDecoder:
             else:
                 self._norm(pending, L["ln1"])
                 self._gemv(self.xn, L["wqkv"], self.qkv)
+            if trace is not None:
+                trace.append(self.x.clone())  # the pending down projection has just been added: the layer's input
             if self.fused_attn:
                 _lib.check(lib.chadq_attn_decode_mqa_fused(self.qkv.data_ptr(), self.pos.data_ptr(), self.rope.data_ptr(),
                                                            self.kcache[li].data_ptr(), self.vcache[li].data_ptr(),
@@ -178,6 +183,8 @@ class QuantDecoder:
                 self._gemv(self.h, L["wd"], self.dn)
             pending = self.dn
         self._norm(pending, self.w["lnf"])
+        if trace is not None:
+            trace.append(self.x.clone())
         self._gemv(self.xn, self.w["emb"], self.logits)
         if self.sampling is None:
             _lib.check(lib.chadq_argmax_f32(self.logits.data_ptr(), c.vocab, self.scratch.data_ptr(), self.token.data_ptr(),
@@ -217,9 +224,22 @@ class QuantDecoder:
         torch.cuda.synchronize()
         self.graph = g
 
+    def _check_range(self, pos: int, n: int, tokens=()) -> None:
+        """The kernels clamp a position to the cache and a token to the table so that nothing is addressed out of
+        bounds, but a clamped step is a wrong step (it overwrites the last cache row and rotates by the wrong angle):
+        refuse on the host what would run past the cache or name a token outside the vocabulary."""
+        if pos < 0 or n < 0 or pos + n > self.cfg.max_ctx:
+            raise ValueError("positions %d..%d do not fit the cache of %d rows" % (pos, pos + n - 1, self.cfg.max_ctx))
+        for t in tokens:
+            if not 0 <= int(t) < self.cfg.vocab:
+                raise ValueError("token %d is outside the vocabulary [0, %d)" % (int(t), self.cfg.vocab))
+
     def feed(self, tokens, pos: int = 0) -> int:
         """Runs the step over a given token sequence starting at position `pos` (the prompt, one token at a time: there
-        is no batched prefill here), filling the caches; returns the token the model proposes after the last one."""
+        is no batched prefill here), filling the caches; returns the token the model proposes after the last one.
+        Raises ValueError if the sequence would run past max_ctx or holds a token outside the vocabulary."""
+        tokens = list(tokens)
+        self._check_range(pos, len(tokens), tokens)
         self.pos.fill_(pos)
         for t in tokens:
             self.token.fill_(int(t))  # overrides the token the previous step proposed
@@ -233,7 +253,8 @@ class QuantDecoder:
 
     def generate(self, first_token: int, pos: int, n: int) -> List[int]:
         """Decodes n tokens starting from `first_token` at position `pos` (the cache holds pos rows): greedy, or sampled
-        as set_sampling() says."""
+        as set_sampling() says.  Raises ValueError if pos + n exceeds max_ctx or first_token is outside the vocabulary."""
+        self._check_range(pos, n, (first_token,))
         self.token.fill_(first_token)
         self.pos.fill_(pos)
         out = []

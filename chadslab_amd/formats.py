@@ -19,6 +19,7 @@ import torch
 
 GROUP = 32
 ZERO_POINT = 8
+FP16_MAX = 65504.0
 
 
 @dataclass
@@ -81,13 +82,20 @@ def pack_int4(q: torch.Tensor) -> torch.Tensor:
 
 
 def quantize_int4_g32(w: torch.Tensor) -> QWeightInt4G32:
-    """fp32 [N,K] -> int4 group-32: scale = absmax/7 per group (stored fp16), q = clamp(rne(w/scale), -8, 7)."""
+    """fp32 [N,K] -> int4 group-32: scale = min(absmax/7, 65504) per group (stored fp16), q = clamp(rne(w/scale), -8, 7).
+    Raises on NaN or infinite weights."""
     w = w.to(torch.float32)
     n, k = w.shape
     if k % GROUP:
         raise ValueError("K must be a multiple of 32")
+    if not bool(torch.isfinite(w).all()):
+        raise ValueError("quantize_int4_g32: the matrix holds NaN or infinite values")
     g = w.reshape(n, k // GROUP, GROUP)
-    s = (g.abs().amax(dim=2) / 7.0).to(torch.float16)
+    # a group whose absmax / 7 exceeds the largest fp16 (65504) keeps that scale and saturates at -8 / 7
+    # the divisor is a tensor on purpose: torch turns a division by a Python scalar on the GPU into a multiplication by
+    # its reciprocal, which is not the correctly rounded quotient a CPU runtime (and the oracle) computes
+    amax = g.abs().amax(dim=2)
+    s = (amax / torch.full_like(amax, 7.0)).clamp(max=FP16_MAX).to(torch.float16)
     sf = s.to(torch.float32)
     sf = torch.where(sf == 0, torch.ones_like(sf), sf)
     q = torch.clamp(torch.round(g / sf[:, :, None]), -8, 7).to(torch.int8).reshape(n, k)
@@ -97,7 +105,10 @@ def quantize_int4_g32(w: torch.Tensor) -> QWeightInt4G32:
 def quantize_int8_row(w: torch.Tensor) -> QWeightInt8:
     """fp32 [N,K] -> int8 per-row: scale = absmax/127 per row (fp32), q = clamp(rne(w/scale), -127, 127)."""
     w = w.to(torch.float32)
-    s = (w.abs().amax(dim=1) / 127.0).to(torch.float32)
+    if not bool(torch.isfinite(w).all()):
+        raise ValueError("quantize_int8_row: the matrix holds NaN or infinite values")
+    amax = w.abs().amax(dim=1)
+    s = (amax / torch.full_like(amax, 127.0)).to(torch.float32)  # a tensor divisor: see quantize_int4_g32
     ss = torch.where(s == 0, torch.ones_like(s), s)
     q = torch.clamp(torch.round(w / ss[:, None]), -127, 127).to(torch.int8)
     return QWeightInt8(q.contiguous(), s.contiguous())

@@ -29,6 +29,17 @@ def _dev(t: torch.Tensor, name: str, dtype: torch.dtype) -> torch.Tensor:
     return t if t.is_contiguous() else t.contiguous()
 
 
+def _out(out: Optional[torch.Tensor], shape, dtype: torch.dtype, device) -> torch.Tensor:
+    """A caller's result tensor, checked before its address goes to the library; a fresh one if none was given."""
+    if out is None:
+        return torch.empty(*shape, dtype=dtype, device=device)
+    if not out.is_cuda or out.device != device:
+        raise ValueError("out must live on %s, got %s" % (device, out.device))
+    if out.dtype != dtype or tuple(out.shape) != tuple(shape) or not out.is_contiguous():
+        raise ValueError("out must be a contiguous %s tensor of shape %s, got %s %s" % (dtype, tuple(shape), out.dtype, tuple(out.shape)))
+    return out
+
+
 def unpack_int4(packed: torch.Tensor) -> torch.Tensor:
     """uint8 [..., K/2] -> int8 [..., K] in [-8,7] (low nibble = even k)."""
     p = _dev(packed, "packed", torch.uint8)
@@ -74,14 +85,14 @@ def qgemv(x: torch.Tensor, qw: QWeight, out: Optional[torch.Tensor] = None) -> t
     if isinstance(qw, QWeightInt4G32):
         x = _dev(x, "x", torch.bfloat16)
         p, s = _dev(qw.packed, "packed", torch.uint8), _dev(qw.scale, "scale", torch.float16)
-        y = out if out is not None else torch.empty(m, qw.N, dtype=torch.float32, device=x.device)
+        y = _out(out, (m, qw.N), torch.float32, x.device)
         _lib.check(lib.chadq_gemv_i4g32(x.data_ptr(), p.data_ptr(), s.data_ptr(), y.data_ptr(), m, qw.N, qw.K,
                                         _stream()), "chadq_gemv_i4g32")
         return y
     if isinstance(qw, QWeightInt8):
         x = _dev(x, "x", torch.float32)
         w, s = _dev(qw.w, "w", torch.int8), _dev(qw.scale, "scale", torch.float32)
-        y = out if out is not None else torch.empty(m, qw.N, dtype=torch.float32, device=x.device)
+        y = _out(out, (m, qw.N), torch.float32, x.device)
         _lib.check(lib.chadq_gemv_i8row(x.data_ptr(), w.data_ptr(), s.data_ptr(), y.data_ptr(), m, qw.N, qw.K,
                                         _stream()), "chadq_gemv_i8row")
         return y
@@ -95,7 +106,7 @@ def qgemm(x: torch.Tensor, qw: QWeight, out: Optional[torch.Tensor] = None) -> t
         raise ValueError("x must be [M,%d], got %s" % (qw.K, tuple(x.shape)))
     x = _dev(x, "x", torch.bfloat16)
     m = x.shape[0]
-    y = out if out is not None else torch.empty(m, qw.N, dtype=torch.bfloat16, device=x.device)
+    y = _out(out, (m, qw.N), torch.bfloat16, x.device)
     if isinstance(qw, QWeightInt4G32):
         p, s = _dev(qw.packed, "packed", torch.uint8), _dev(qw.scale, "scale", torch.float16)
         _lib.check(lib.chadq_gemm_i4g32_bf16(x.data_ptr(), p.data_ptr(), s.data_ptr(), y.data_ptr(), m, qw.N, qw.K,
@@ -138,7 +149,7 @@ def moe_route(logits: torch.Tensor, top_k: int = 2, renorm: bool = True):
     return idx, w
 
 
-_moe_ws = {}  # (device, bytes) -> workspace tensor, reused between calls
+_moe_ws = {}  # (device, stream, bytes) -> workspace tensor, reused between calls on that stream
 
 
 def moe_ffn(x: torch.Tensor, logits: torch.Tensor, experts, *, top_k: int = 2, renorm: bool = True) -> torch.Tensor:
@@ -165,7 +176,11 @@ def moe_ffn(x: torch.Tensor, logits: torch.Tensor, experts, *, top_k: int = 2, r
     need = lib.chadq_moe_ffn_i4g32_workspace_bytes(t, h, f, e, top_k)
     if need == 0:
         raise ValueError("unsupported MoE sizes T=%d H=%d F=%d E=%d top_k=%d" % (t, h, f, e, top_k))
-    key = (x.device, need)
+    # The workspace holds the router's output and every intermediate of the call, so two calls in flight at once must
+    # not share one: calls on one stream are ordered and reuse theirs, another stream gets its own.  A graph captured
+    # on a stream keeps using that stream's workspace on every replay: do not run eager calls of the same sizes on the
+    # capture stream while a replay is in flight.
+    key = (x.device, _stream(), need)
     ws = _moe_ws.get(key)
     if ws is None:
         ws = _moe_ws[key] = torch.empty(need, dtype=torch.uint8, device=x.device)

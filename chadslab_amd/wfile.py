@@ -93,10 +93,25 @@ def read_header(path: str) -> Dict:
         return json.loads(f.read(hlen).decode("utf-8"))
 
 
+SLAB_BYTES = 64 << 20
+
+
+def _copy_out(m: np.ndarray, shape, device) -> torch.Tensor:
+    """The mapped flat array `m` as a tensor of `shape` on `device`, copied in slabs of at most 64 MiB so that the
+    host never holds more than one slab of it outside the page cache."""
+    n = m.shape[0]
+    out = torch.empty(n, dtype=torch.from_numpy(np.empty(0, dtype=m.dtype)).dtype, device=device)
+    step = max(1, SLAB_BYTES // max(1, m.dtype.itemsize))
+    for a in range(0, n, step):
+        b = min(n, a + step)
+        out[a:b].copy_(torch.from_numpy(np.array(m[a:b])))  # np.array: the slab's one host copy (the map is read-only)
+    return out.reshape(shape)
+
+
 def load(path: str, device="cpu") -> Dict[str, Entry]:
-    """Memory-maps `path` and returns name -> QWeightInt4G32 / QWeightInt8 / tensor on `device`.  With device="cpu"
-    the tensors are copies (the map is closed on return); with a GPU device each array is copied straight from the
-    map to the device."""
+    """Memory-maps `path` and returns name -> QWeightInt4G32 / QWeightInt8 / tensor on `device`.  Every array is
+    copied out of the map in slabs of 64 MiB (to the GPU for a GPU device), so a multi-GB file is never held whole
+    in host memory; the map is closed on return."""
     hdr = read_header(path)
     size = np.memmap(path, dtype=np.uint8, mode="r").shape[0]
     out: Dict[str, Entry] = {}
@@ -107,8 +122,8 @@ def load(path: str, device="cpu") -> Dict[str, Entry]:
             n = int(np.prod(d["shape"])) if d["shape"] else 1
             if d["offset"] % ALIGN or d["offset"] + n * dt.itemsize > size or n * dt.itemsize != d["nbytes"]:
                 raise ValueError("%s: array %s/%s does not fit the file" % (path, name, an))
-            m = np.memmap(path, dtype=dt, mode="r", offset=d["offset"], shape=tuple(d["shape"]))
-            arrs[an] = torch.from_numpy(np.array(m)).to(device)  # np.array: one host copy, then the device copy
+            m = np.memmap(path, dtype=dt, mode="r", offset=d["offset"], shape=(n,))
+            arrs[an] = _copy_out(m, tuple(d["shape"]), device)
             del m
         if t["kind"] == "i4g32":
             out[name] = QWeightInt4G32(arrs["packed"], arrs["scale"])

@@ -31,6 +31,9 @@ accumulation case, and the independent scalar C twin in chadq_oracle.c.
 """
 from __future__ import annotations
 
+import os
+from concurrent.futures import ThreadPoolExecutor
+
 import numpy as np
 
 GROUP = 32          # int4 scale group length along K
@@ -118,9 +121,26 @@ def qgemm_int4g32_f64(x_bf16: np.ndarray, wp: np.ndarray, scale_f16: np.ndarray)
     return x @ dequant_int4g32(wp, scale_f16).astype(np.float64).T
 
 
+CHUNK_ELEMS = 1 << 20   # weights dequantised at a time: a worker's fp32 copy (4 MB) stays in its cache
+WORKERS = min(8, os.cpu_count() or 1)
+
+
 def qgemv_int4g32(x_bf16: np.ndarray, wp: np.ndarray, scale_f16: np.ndarray) -> np.ndarray:
-    """Configs 1: x bf16 bits [M,K] -> fp32 [M,N]; dequantise to fp32, then an fp32 matmul."""
-    return bf16_to_f32(x_bf16) @ dequant_int4g32(wp, scale_f16).T
+    """Configs 1: x bf16 bits [M,K] -> fp32 [M,N]; dequantise to fp32, then an fp32 matmul.  A matrix of more than
+    CHUNK_ELEMS weights is handled in blocks of whole rows, a few at a time on worker threads (numpy releases the
+    interpreter lock inside its loops): each output column depends on its own weight row only, so the blocks are
+    independent and the result does not depend on how many workers there are."""
+    x = bf16_to_f32(x_bf16)
+    n, k = wp.shape[0], wp.shape[1] * 2
+    rows = max(1, CHUNK_ELEMS // max(1, k))
+    if n <= rows:
+        return x @ dequant_int4g32(wp, scale_f16).T
+
+    def block(r):
+        return x @ dequant_int4g32(wp[r: r + rows], scale_f16[r: r + rows]).T
+
+    with ThreadPoolExecutor(WORKERS) as ex:
+        return np.concatenate(list(ex.map(block, range(0, n, rows))), axis=1)
 
 
 def qgemm_int4g32_bf16(x_bf16, wp, scale_f16) -> np.ndarray:
@@ -195,11 +215,11 @@ def moe_qffn(x_bf16, logits, experts, top_k: int = 2, renorm: bool = True) -> np
 
 # --------------------------------------------------------------------------- quantiser (next-row helper)
 def quantize_int4_g32(w: np.ndarray):
-    """fp32 [N,K] -> (packed uint8 [N,K/2], scale fp16 [N,K/32]); absmax/7 per group, RNE, clamp to [-8,7]."""
+    """fp32 [N,K] -> (packed uint8 [N,K/2], scale fp16 [N,K/32]); min(absmax/7, 65504) per group, RNE, clamp to [-8,7]."""
     w = np.asarray(w, dtype=np.float32)
     n, k = w.shape
     g = w.reshape(n, k // GROUP, GROUP)
-    s = (np.abs(g).max(axis=2) / np.float32(7)).astype(np.float16)
+    s = np.minimum(np.abs(g).max(axis=2) / np.float32(7), np.float32(65504)).astype(np.float16)  # largest fp16: no inf scale
     sf = s.astype(np.float32)
     sf_safe = np.where(sf == 0, np.float32(1), sf)
     q = np.clip(np.rint(g / sf_safe[:, :, None]), -8, 7).astype(np.int8).reshape(n, k)
@@ -250,36 +270,47 @@ def gelu_tanh(x):
     return (0.5 * x * (1.0 + np.tanh(np.float32(0.7978845608028654) * (x + np.float32(0.044715) * x * x * x)))).astype(np.float32)
 
 
+def decode_layer(L, x, pos, kcache, vcache, hq, dh, eps=1e-6, base=10000.0):
+    """One decoder layer on the fp32 residual vector x [d]: attention block, then the gated FFN block.  L: {"ln1",
+    "wqkv", "wo", "ln2", "wgu", "wd"} with weights as (packed, scale) tuples; kcache/vcache: this layer's bf16 bit
+    arrays [max_ctx, dh], row `pos` is written.  Returns the residual vector after the layer."""
+    xn = f32_to_bf16(rmsnorm(x, L["ln1"], eps))[None, :]
+    qkv = qgemv_int4g32(xn, *L["wqkv"])[0]
+    q = rope_rotate_half(qkv[: hq * dh].reshape(hq, dh), pos, base)
+    k = rope_rotate_half(qkv[hq * dh: (hq + 1) * dh], pos, base)
+    v = qkv[(hq + 1) * dh:]
+    kcache[pos] = f32_to_bf16(k)
+    vcache[pos] = f32_to_bf16(v)
+    kk = bf16_to_f32(kcache[: pos + 1])
+    vv = bf16_to_f32(vcache[: pos + 1])
+    sc = (q @ kk.T) / np.float32(np.sqrt(dh))
+    sc = sc - sc.max(axis=-1, keepdims=True)
+    p = np.exp(sc)
+    p = p / p.sum(axis=-1, keepdims=True)
+    att = f32_to_bf16((p @ vv).astype(np.float32)).reshape(1, hq * dh)
+    x = x + qgemv_int4g32(att, *L["wo"])[0]
+    xn = f32_to_bf16(rmsnorm(x, L["ln2"], eps))[None, :]
+    gu = qgemv_int4g32(xn, *L["wgu"])[0]
+    f = gu.shape[0] // 2
+    h = f32_to_bf16(gelu_tanh(gu[:f]) * gu[f:])[None, :]
+    return x + qgemv_int4g32(h, *L["wd"])[0]
+
+
+def decode_logits(model, x, eps=1e-6):
+    """Final norm and the tied output table on the residual vector x [d]: fp32 logits [V]."""
+    xn = f32_to_bf16(rmsnorm(x, model["lnf"], eps))[None, :]
+    return qgemv_int4g32(xn, *model["emb"])[0]
+
+
 def decode_step(model, token, pos, kcache, vcache, hq, dh, eps=1e-6, base=10000.0):
     """One token of a decoder-only transformer on int4 group-32 weights.  model: {"layers": [{"ln1","wqkv",
     "wo","ln2","wgu","wd"}], "lnf", "emb"} with weights as (packed, scale) tuples.  kcache/vcache: per layer
     bf16 bit arrays [max_ctx, dh], row `pos` is written.  Returns fp32 logits [V]."""
     ep, es = model["emb"]
-    d = ep.shape[1] * 2
     x = dequant_int4g32(ep[token:token + 1], es[token:token + 1])[0]
     for li, L in enumerate(model["layers"]):
-        xn = f32_to_bf16(rmsnorm(x, L["ln1"], eps))[None, :]
-        qkv = qgemv_int4g32(xn, *L["wqkv"])[0]
-        q = rope_rotate_half(qkv[: hq * dh].reshape(hq, dh), pos, base)
-        k = rope_rotate_half(qkv[hq * dh: (hq + 1) * dh], pos, base)
-        v = qkv[(hq + 1) * dh:]
-        kcache[li][pos] = f32_to_bf16(k)
-        vcache[li][pos] = f32_to_bf16(v)
-        kk = bf16_to_f32(kcache[li][: pos + 1])
-        vv = bf16_to_f32(vcache[li][: pos + 1])
-        sc = (q @ kk.T) / np.float32(np.sqrt(dh))
-        sc = sc - sc.max(axis=-1, keepdims=True)
-        p = np.exp(sc)
-        p = p / p.sum(axis=-1, keepdims=True)
-        att = f32_to_bf16((p @ vv).astype(np.float32)).reshape(1, hq * dh)
-        x = x + qgemv_int4g32(att, *L["wo"])[0]
-        xn = f32_to_bf16(rmsnorm(x, L["ln2"], eps))[None, :]
-        gu = qgemv_int4g32(xn, *L["wgu"])[0]
-        f = gu.shape[0] // 2
-        h = f32_to_bf16(gelu_tanh(gu[:f]) * gu[f:])[None, :]
-        x = x + qgemv_int4g32(h, *L["wd"])[0]
-    xn = f32_to_bf16(rmsnorm(x, model["lnf"], eps))[None, :]
-    return qgemv_int4g32(xn, ep, es)[0]
+        x = decode_layer(L, x, pos, kcache[li], vcache[li], hq, dh, eps, base)
+    return decode_logits(model, x, eps)
 
 
 def sample_topk(v: np.ndarray, k: int, temperature: float, u: float) -> int:

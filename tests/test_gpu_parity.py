@@ -156,6 +156,25 @@ def test_gemv_int4_tall_matrices(ops, m, n, k):
     assert np.isfinite(y).all() and O.rel_l2(y, O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_F32
 
 
+@pytest.mark.parametrize("m", [1, 4])
+def test_gemv_int4_output_table_256000_rows(ops, m):
+    # the decode step's output projection: 256000 rows of K = 2048 (the tallest matrix the benchmark has); the float64
+    # truth and the integer brute force are formed 32000 rows at a time to keep the host's copies small
+    from chadslab_amd import QWeightInt4G32
+
+    n, k, step = 256000, 2048, 32000
+    packed, s, xb, qw = i4_case(4100 + m, m, n, k)
+    y = ops.qgemv(bf16_tensor(xb), qw).cpu().numpy()
+    assert y.shape == (m, n) and np.isfinite(y).all()
+    want = np.concatenate([O.qgemm_int4g32_f64(xb, packed[r: r + step], s[r: r + step]) for r in range(0, n, step)], axis=1)
+    assert O.rel_l2(y, want) <= TOL_F32
+    xi = O.f32_to_bf16(rng(4102).integers(-8, 9, (m, k)).astype(np.float32))
+    yi = ops.qgemv(bf16_tensor(xi), QWeightInt4G32(qw.packed, torch.ones_like(qw.scale))).cpu().numpy()
+    xf = O.bf16_to_f32(xi).astype(np.float64)  # small integers: float64 sums of their products are exact
+    brute = np.concatenate([xf @ O.unpack_int4(packed[r: r + step]).astype(np.float64).T for r in range(0, n, step)], axis=1)
+    assert np.abs(brute).max() < 2 ** 24 and np.array_equal(yi, brute.astype(np.float32))
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 14336, 4096), (2, 14336, 4096), (8, 512, 4096), (4, 96, 256), (2, 40, 96)])
 def test_gemv_int4_integer_accumulation_bit_exact(ops, m, n, k):
     from chadslab_amd import QWeightInt4G32
