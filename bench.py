@@ -29,11 +29,25 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16
-# HBM bytes per launch of the headline kernel from hardware counters (FETCH_SIZE, WRITE_SIZE, each scaled by what a
-# 256 MiB copy reads for it); the counter runs are summarised in profiles/gemv_i4g32_m1_config1_hbm_traffic.txt
-GEMV_M1_TRAFFIC_BYTES = 33278000
 N_COPIES = 12
 SEG = 48                     # launches per captured graph
+
+
+def profile_figures():
+    """(HBM bytes per launch of the headline kernel from hardware counters, the kernel's name) as the committed
+    profile summaries state them: profiles/gemv_i4g32_m1_config1_hbm_traffic.txt carries a line
+    `roofline.traffic = <bytes>` and a table row naming the kernel.  Whoever refreshes the counter runs edits those
+    two lines and nothing here; (None, None) if the summary is missing."""
+    import re
+
+    path = os.path.join(ROOT, "profiles", "gemv_i4g32_m1_config1_hbm_traffic.txt")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, None
+    t = re.search(r"^roofline\.traffic\s*=\s*([0-9,]+)", text, re.M)
+    k = re.search(r"^roofline\.kernel\s*=\s*(\S+)", text, re.M)
+    return (int(t.group(1).replace(",", "")) if t else None), (k.group(1) if k else None)
 
 
 def parse():
@@ -77,10 +91,14 @@ def main():
         return t.view(torch.int16).cpu().numpy().view(np.uint16)
 
     def run_steps(fn, steps, warmup):
-        """fn(i) launches step i on the current stream.  Returns (us per step from HIP events, wall us per step)."""
+        """fn(i) launches step i on the current stream.  Returns (us per step from HIP events, wall us per step,
+        launches per replayed graph).  The start event is recorded behind one more untimed replay that is already
+        queued, so the timed replays are submitted while the GPU is still busy: the cost of getting a graph launch
+        to an idle GPU is then not spread over the timed steps, however few they are."""
+        seg = min(SEG, steps)
         with torch.cuda.stream(stream):
             graphs = {}
-            for length in sorted({min(SEG, steps), steps % SEG} - {0}):
+            for length in sorted({seg, steps % seg} - {0}):
                 for i in range(length):
                     fn(i)
                 torch.cuda.synchronize()
@@ -89,23 +107,23 @@ def main():
                     for i in range(length):
                         fn(i)
                 graphs[length] = g
-            full, rem = divmod(steps, min(SEG, steps))
-            wfull = max(1, warmup // min(SEG, steps))
-            for _ in range(wfull):
-                graphs[min(SEG, steps)].replay()
+            full, rem = divmod(steps, seg)
+            for _ in range(max(1, warmup // seg)):
+                graphs[seg].replay()
             torch.cuda.synchronize()
             a = torch.cuda.Event(enable_timing=True)
             b = torch.cuda.Event(enable_timing=True)
             t0 = time.perf_counter()
+            graphs[seg].replay()  # untimed: keeps the GPU busy while the timed replays are submitted
             a.record(stream)
             for _ in range(full):
-                graphs[min(SEG, steps)].replay()
+                graphs[seg].replay()
             if rem:
                 graphs[rem].replay()
             b.record(stream)
             torch.cuda.synchronize()
             t1 = time.perf_counter()
-        return a.elapsed_time(b) * 1000.0 / steps, (t1 - t0) * 1e6 / steps
+        return a.elapsed_time(b) * 1000.0 / steps, (t1 - t0) * 1e6 / (steps + seg), seg
 
     if args.calibration_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -142,20 +160,20 @@ def main():
         x = torch.from_numpy(x_np[m]).to(torch.bfloat16).to(dev)
         y = torch.empty(m, N, dtype=torch.float32, device=dev)
         steps = args.steps if m == 1 else min(args.steps, n_side[0])
-        us, wall = run_steps(lambda i: ops.qgemv(x, copies[i % N_COPIES], out=y), steps, args.warmup)
-        results[m] = (us, wall, steps)
+        us, wall, seg_used = run_steps(lambda i: ops.qgemv(x, copies[i % N_COPIES], out=y), steps, args.warmup)
+        results[m] = (us, wall, steps, seg_used)
         if m == 1:
             from oracle import chadq_oracle as O  # the checker, used once outside the timed region
 
             parity["gemv_i4g32_m1_rel_l2_vs_f64"] = O.rel_l2(y.cpu().numpy(), O.qgemm_int4g32_f64(bits(x), packed, scale))
-    us1, wall1, steps1 = results[1]
+    us1, wall1, steps1, seg1 = results[1]
     achieved = gemv_bytes(1) / us1 * 1e-3  # GB/s
 
     extras = {}
     if "gemv" in want:
         x1 = torch.from_numpy(x_np[1]).to(torch.bfloat16).to(dev)
         y1 = torch.empty(1, N, dtype=torch.float32, device=dev)
-        us_hot, _ = run_steps(lambda i: ops.qgemv(x1, base, out=y1), *n_side)
+        us_hot = run_steps(lambda i: ops.qgemv(x1, base, out=y1), *n_side)[0]
         extras["gemv_i4g32"] = {
             "M%d" % m: {"us": round(results[m][0], 3), "GBps": round(gemv_bytes(m) / results[m][0] * 1e-3, 1),
                         "frac_hbm_peak": round(gemv_bytes(m) / results[m][0] * 1e-3 / HBM_PEAK_GBS, 4)}
@@ -164,22 +182,28 @@ def main():
         extras["gemv_i4g32"]["M1_same_buffer_every_step"] = {
             "us": round(us_hot, 3), "GBps": round(gemv_bytes(1) / us_hot * 1e-3, 1),
             "note": "weights served by the 256 MB last-level cache, not HBM; not a roofline figure"}
-        # what this machine delivers for a cold read of the same number of bytes with the same access shape and no
-        # arithmetic: the practical ceiling next to which the GEMV's time should be read
-        lib = _lib.load()
-        nread = gemv_bytes(1) // 16384 * 16384
-        flat = [torch.empty(nread, dtype=torch.uint8, device=dev).fill_(i + 1) for i in range(N_COPIES)]
-        pout = torch.empty(nread // 16384, dtype=torch.int32, device=dev)
+        # what this machine delivers for a cold read of the same number of bytes and no arithmetic (bench_probe.so,
+        # built from bench_probe.hip): the practical ceiling next to which the GEMV's time should be read
+        import ctypes
 
-        def probe(i):
-            _lib.check(lib.chadq_probe_read(flat[i % N_COPIES].data_ptr(), nread, pout.data_ptr(),
-                                            torch.cuda.current_stream().cuda_stream), "chadq_probe_read")
+        probe_path = os.path.join(ROOT, "bench_probe.so")
+        if os.path.exists(probe_path):
+            plib = ctypes.CDLL(probe_path)
+            plib.bench_probe_read.restype = ctypes.c_int
+            plib.bench_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+            nread = gemv_bytes(1) // 16384 * 16384
+            flat = [torch.empty(nread, dtype=torch.uint8, device=dev).fill_(i + 1) for i in range(N_COPIES)]
+            pout = torch.empty(nread // 16384, dtype=torch.int32, device=dev)
 
-        us_rd, _ = run_steps(probe, *n_side)
-        extras["gemv_i4g32"]["cold_read_same_bytes"] = {
-            "us": round(us_rd, 3), "GBps": round(nread / us_rd * 1e-3, 1), "bytes": int(nread),
-            "note": "loads only (chadq_probe_read), rotating buffers: the machine's ceiling for a read of this size"}
-        del flat, pout
+            def probe(i):
+                if plib.bench_probe_read(flat[i % N_COPIES].data_ptr(), nread, pout.data_ptr(), torch.cuda.current_stream().cuda_stream):
+                    raise RuntimeError("bench_probe_read failed")
+
+            us_rd = run_steps(probe, *n_side)[0]
+            extras["gemv_i4g32"]["cold_read_same_bytes"] = {
+                "us": round(us_rd, 3), "GBps": round(nread / us_rd * 1e-3, 1), "bytes": int(nread),
+                "note": "loads only (bench_probe.hip), rotating buffers: the machine's ceiling for a read of this size"}
+            del flat, pout
     del copies
 
     if "int8" in want:
@@ -191,7 +215,7 @@ def main():
         s0 = torch.from_numpy(r0.uniform(0.001, 0.02, N0).astype(np.float32)).to(dev)
         c0 = [QWeightInt8(w0.clone(), s0.clone()) for _ in range(N_COPIES)]
         y0 = torch.empty(1, N0, dtype=torch.float32, device=dev)
-        us0, _ = run_steps(lambda i: ops.qgemv(x0, c0[i % N_COPIES], out=y0), *n_side)
+        us0 = run_steps(lambda i: ops.qgemv(x0, c0[i % N_COPIES], out=y0), *n_side)[0]
         b0 = N0 * K0 + N0 * 4 + K0 * 4 + N0 * 4
         extras["gemv_i8row_config0"] = {"us": round(us0, 3), "GBps": round(b0 / us0 * 1e-3, 1),
                                         "frac_hbm_peak": round(b0 / us0 * 1e-3 / HBM_PEAK_GBS, 4)}
@@ -209,26 +233,33 @@ def main():
                          torch.from_numpy(r2.uniform(0.001, 0.02, N2).astype(np.float32)).to(dev))
         flop = 2.0 * M2 * N2 * K2
         for name, qw in (("gemm_i4g32_config2", q4), ("gemm_i8row_config2", q8)):
-            usg, _ = run_steps(lambda i: ops.qgemm(x2, qw, out=y2), *n_gemm)
+            usg = run_steps(lambda i: ops.qgemm(x2, qw, out=y2), *n_gemm)[0]
             extras[name] = {"us": round(usg, 3), "TFLOPs": round(flop / usg * 1e-6, 1),
                             "frac_bf16_mfma_peak": round(flop / usg * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
         # context: the vendor library's plain bf16 GEMM (no dequantisation) on the same shape, through torch.matmul
         wb16 = torch.randn(N2, K2, device=dev).to(torch.bfloat16)
         yt = torch.empty(M2, N2, dtype=torch.bfloat16, device=dev)
-        ust, _ = run_steps(lambda i: torch.matmul(x2, wb16.t(), out=yt), *n_gemm)
+        ust = run_steps(lambda i: torch.matmul(x2, wb16.t(), out=yt), *n_gemm)[0]
         extras["gemm_bf16_library_same_shape"] = {"us": round(ust, 3), "TFLOPs": round(flop / ust * 1e-6, 1),
                                                   "note": "torch.matmul on bf16 weights (hipBLASLt/rocBLAS): context, not this build's kernel"}
-        del wb16, yt
-
-        # the kernel's asymptote at a larger M (not a benchmark config: extra, labelled as such)
+        # many rows (not a benchmark configuration: extra, labelled as such): the 256 x 256 tile kernel, and beside it the
+        # vendor library's plain bf16 GEMM on the same shape and on random data, which is what the matrix cores of this
+        # machine sustain once their power draw sets the clock (the same call on zeros runs half as long)
         M2b = 4096
         x2b = torch.randn(M2b, K2, device=dev).to(torch.bfloat16)
         y2b = torch.empty(M2b, N2, dtype=torch.bfloat16, device=dev)
-        usb, _ = run_steps(lambda i: ops.qgemm(x2b, q4, out=y2b), max(8, n_gemm[0] // 8), 4)
-        extras["gemm_i4g32_M4096_extra"] = {"us": round(usb, 2), "TFLOPs": round(2.0 * M2b * N2 * K2 / usb * 1e-6, 1),
-                                            "frac_bf16_mfma_peak": round(2.0 * M2b * N2 * K2 / usb * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4),
-                                            "note": "same kernel at M=4096, N=K=4096: not a benchmark configuration"}
+        nbig = (max(8, n_gemm[0] // 8), 4)
+        usb = run_steps(lambda i: ops.qgemm(x2b, q4, out=y2b), *nbig)[0]
+        flopb = 2.0 * M2b * N2 * K2
+        extras["gemm_i4g32_M4096_extra"] = {"us": round(usb, 2), "TFLOPs": round(flopb / usb * 1e-6, 1),
+                                            "frac_bf16_mfma_peak": round(flopb / usb * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                            "note": "M=4096, N=K=4096 (large-tile kernel): not a benchmark configuration"}
+        ustb = run_steps(lambda i: torch.matmul(x2b, wb16.t(), out=y2b), *nbig)[0]
+        extras["gemm_bf16_library_M4096_extra"] = {"us": round(ustb, 2), "TFLOPs": round(flopb / ustb * 1e-6, 1),
+                                                   "frac_bf16_mfma_peak": round(flopb / ustb * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                                   "note": "torch.matmul on bf16 weights, random data: context, not this build's kernel"}
+        del wb16, yt
         del x2, y2, q4, q8, p2, s2, x2b, y2b
     if "moe" in want:
         # config 3: mixture-of-experts FFN, 8 experts, top-2, 256 tokens (weights random bytes: timing only, parity
@@ -357,6 +388,7 @@ def main():
             "host_cpus": os.cpu_count(),
         }
 
+    traffic_bytes, kernel_name = profile_figures()
     out = {
         "metric": "int4 GEMV HBM GB/s (% peak) + dequant-GEMM TFLOP/s (% MFMA peak), 1 GPU",
         "value": round(achieved, 1),
@@ -371,11 +403,11 @@ def main():
         "dtype": "bf16 x int4 -> fp32 accumulate",
         "data": "synthetic",
         "config": {"workload": "config 1: int4 group-32 decode GEMV, M=1, W [14336,4096], x bf16, y fp32",
-                   "M": 1, "N": N, "K": K, "weight_copies_rotated": N_COPIES, "launch": "HIP graph replay, %d launches per graph" % SEG,
+                   "M": 1, "N": N, "K": K, "weight_copies_rotated": N_COPIES, "launch": "HIP graph replay, %d launches per graph" % seg1,
                    "algorithmic_bytes_per_launch": gemv_bytes(1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_M1_TRAFFIC_BYTES,
-                     "kernel": "gemv_i4g32_mfma_kernel<1,2,16,1,4,4096>", "wall_clock_us_per_step": round(wall1, 3)},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_bytes,
+                     "kernel": kernel_name, "wall_clock_us_per_step": round(wall1, 3)},
         "cpu_baseline": cpu,
         "parity": parity,
         "extras": extras,

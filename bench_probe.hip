@@ -1,0 +1,40 @@
+// A measuring aid for bench.py, not part of libchadq: a read of `bytes` bytes with the decode GEMV's per-wave footprint
+// and nothing else (every wave owns 16 KiB, keeps four 1-KiB loads in flight, folds what it read across its lanes and
+// stores one word), so that the benchmark can report what this machine delivers for a cold read of the same size next
+// to the GEMV's own time.  Built into bench_probe.so next to bench.py by __graft_entry__.build().
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+constexpr int PROBE_WAVE_BYTES = 16384;  // per wave: 16 loads of 1 KiB, like a wave of the GEMV at K = 4096
+
+__global__ __launch_bounds__(256) void probe_read_kernel(const uint8_t *__restrict__ src, size_t nwaves, uint32_t *__restrict__ out) {
+    const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (wave >= nwaves) return;
+    const uint8_t *p = src + wave * PROBE_WAVE_BYTES + lane * 16;
+    u32x4 v[16];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p + i * 1024));
+    uint32_t acc = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        asm volatile("" : "+v"(v[i]));  // wait for exactly this load
+        if (i + 4 < 16) v[i + 4] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p + (i + 4) * 1024));
+        acc ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    }
+    for (int o = 1; o < 64; o <<= 1) acc ^= (uint32_t)__shfl_xor((int)acc, o, 64);
+    if (lane == 0) out[wave] = acc;
+}
+
+// Reads the first bytes / 16384 * 16384 bytes of src (16-byte aligned device memory) and stores one word per 16 KiB to
+// out.  Returns 0, or the HIP error code of the launch.
+extern "C" int bench_probe_read(const void *src, int64_t bytes, uint32_t *out, void *stream) {
+    if (!src || !out || bytes < 0 || (reinterpret_cast<uintptr_t>(src) & 15u)) return -1;
+    const size_t nwaves = (size_t)bytes / PROBE_WAVE_BYTES;
+    if (nwaves == 0) return 0;
+    hipLaunchKernelGGL(probe_read_kernel, dim3((unsigned)((nwaves + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<const uint8_t *>(src), nwaves, out);
+    return (int)hipGetLastError();
+}

@@ -9,7 +9,10 @@ import ctypes
 from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "libchadq.so"
+import os
+
+# CHADQ_LIB names another build of the library to load instead of the in-tree one (comparing two builds on one box)
+LIB_PATH = Path(os.environ.get("CHADQ_LIB") or (Path(__file__).resolve().parent / "libchadq.so"))
 
 # name -> (restype, argtypes); mirrors include/chadq.h one to one
 SIGNATURES = {
@@ -46,7 +49,6 @@ SIGNATURES = {
                                                    c_void_p]),
     "chadq_geglu_bf16": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     "chadq_argmax_f32": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
-    "chadq_probe_read": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "chadq_sample_topk_f32": (c_int, [c_void_p, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
 }
 

@@ -73,7 +73,6 @@ int attn_mqa_fused_static_launch(const float *, const int32_t *, const float *, 
                                  hipStream_t);
 int attn_mqa_fused_static_max_ctx();
 int argmax_launch(const float *, int, float *, int32_t *, int32_t *, int32_t *, int, hipStream_t);
-int probe_read_launch(const uint8_t *, size_t, uint32_t *, hipStream_t);
 int sample_topk_launch(const float *, int, int, float, const float *, float *, int32_t *, int32_t *, int32_t *, int, hipStream_t);
 
 }  // namespace chadq
@@ -363,14 +362,6 @@ int chadq_sample_topk_f32(const float *v, int n, int k, float temperature, const
     float *cv = reinterpret_cast<float *>(workspace);
     int32_t *ci = reinterpret_cast<int32_t *>(cv + 96 * 64);
     return sample_topk_launch(v, n, k, temperature, u, cv, ci, token, pos, advance, st);
-}
-
-int chadq_probe_read(const void *src, int64_t bytes, uint32_t *out, void *stream) {
-    ENTER();
-    CHADQ_REQUIRE(bytes >= 0, CHADQ_ERR_SHAPE, "chadq_probe_read: bytes=%lld is negative", (long long)bytes);
-    CHADQ_REQUIRE(src && out, CHADQ_ERR_NULL, "chadq_probe_read: null pointer");
-    CHADQ_REQUIRE((reinterpret_cast<uintptr_t>(src) & 15u) == 0, CHADQ_ERR_ALIGN, "chadq_probe_read: src must be 16-byte aligned");
-    return probe_read_launch(reinterpret_cast<const uint8_t *>(src), (size_t)bytes, out, st);
 }
 
 }  // extern "C"

@@ -135,6 +135,28 @@ __device__ __forceinline__ void unpack8_magic_r(uint32_t w, uint32_t mask_reg, u
     p[3] = and_or(w >> 12, mask_reg, magic_reg);
 }
 
+// 8 nibbles of word `w` (u0 lowest) -> 8 bf16 of (u-8)*s in k order, the int4 group-32 dequantisation the matrix-core
+// kernels share.  fp16 magic: 0x6400|u reads 1024+u, and a nibble left in bits 7:4 reads 1024+16u; one fp32 FMA per
+// element removes the offset and applies the scale, then RNE to bf16.  Callers pass s16 = s/16, c0 = -1032 s,
+// c1 = -72 s, and mlo = 0x000F000F, mhi = 0x00F000F0, magic = 0x64006400 in registers so that each pair of nibbles
+// costs one v_and_or_b32.
+__device__ __forceinline__ bf16x8 dequant8_i4(uint32_t w, float s, float s16, float c0, float c1, uint32_t mlo, uint32_t mhi,
+                                              uint32_t magic) {
+    const f16x2 h0 = as_f16x2(and_or(w, mlo, magic));   // u0, u4
+    const f16x2 h1 = as_f16x2(and_or(w, mhi, magic));   // 16*u1, 16*u5
+    const uint32_t w8 = w >> 8;
+    const f16x2 h2 = as_f16x2(and_or(w8, mlo, magic));  // u2, u6
+    const f16x2 h3 = as_f16x2(and_or(w8, mhi, magic));  // 16*u3, 16*u7
+    const float f0 = __builtin_fmaf((float)h0.x, s, c0), f4 = __builtin_fmaf((float)h0.y, s, c0);
+    const float f1 = __builtin_fmaf((float)h1.x, s16, c1), f5 = __builtin_fmaf((float)h1.y, s16, c1);
+    const float f2 = __builtin_fmaf((float)h2.x, s, c0), f6 = __builtin_fmaf((float)h2.y, s, c0);
+    const float f3 = __builtin_fmaf((float)h3.x, s16, c1), f7 = __builtin_fmaf((float)h3.y, s16, c1);
+    const u32x4 r = {pack_bf16_rne(f0, f1), pack_bf16_rne(f2, f3), pack_bf16_rne(f4, f5), pack_bf16_rne(f6, f7)};
+    bf16x8 o;
+    __builtin_memcpy(&o, &r, 16);
+    return o;
+}
+
 // A constant the optimiser must keep in a vector register.
 __device__ __forceinline__ uint32_t vgpr_const(uint32_t v) {
     uint32_t r;

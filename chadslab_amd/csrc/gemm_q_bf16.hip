@@ -19,6 +19,7 @@
 // The MFMA k-slot of a lane is free to choose as long as A and B agree: slot group kq covers the kq-th
 // 16-byte weight load, and step t of that load is its t-th 8-k word.
 // The four partial tiles are summed through LDS at the end, rounded to bf16 (RNE) and stored coalesced.
+#include <cstdlib>
 #include <type_traits>
 
 #include "chadq_common.h"
@@ -28,26 +29,6 @@ namespace chadq {
 struct FmtI4G32 {
     static constexpr int KL = 32;  // k per 16-byte weight load
     typedef uint16_t scale_t;
-    // 8 nibbles of word `w` -> 8 bf16 of (u-8)*s, k order.  fp16 magic: 0x6400|u = 1024+u, and a nibble left
-    // in bits 7:4 reads as 1024+16u; one fp32 FMA per element removes the offsets and applies the scale.
-    // mlo = 0x000F000F, mhi = 0x00F000F0 and magic = 0x64006400 are handed over in registers so that each
-    // pair of nibbles costs one v_and_or_b32.
-    __device__ static __forceinline__ bf16x8 dequant(uint32_t w, float s, float s16, float c0, float c1, uint32_t mlo,
-                                                     uint32_t mhi, uint32_t magic) {
-        const f16x2 h0 = as_f16x2(and_or(w, mlo, magic));  // u0, u4
-        const f16x2 h1 = as_f16x2(and_or(w, mhi, magic));  // 16*u1, 16*u5
-        const uint32_t w8 = w >> 8;
-        const f16x2 h2 = as_f16x2(and_or(w8, mlo, magic));  // u2, u6
-        const f16x2 h3 = as_f16x2(and_or(w8, mhi, magic));  // 16*u3, 16*u7
-        const float f0 = __builtin_fmaf((float)h0.x, s, c0), f4 = __builtin_fmaf((float)h0.y, s, c0);
-        const float f1 = __builtin_fmaf((float)h1.x, s16, c1), f5 = __builtin_fmaf((float)h1.y, s16, c1);
-        const float f2 = __builtin_fmaf((float)h2.x, s, c0), f6 = __builtin_fmaf((float)h2.y, s, c0);
-        const float f3 = __builtin_fmaf((float)h3.x, s16, c1), f7 = __builtin_fmaf((float)h3.y, s16, c1);
-        const u32x4 r = {pack_bf16_rne(f0, f1), pack_bf16_rne(f2, f3), pack_bf16_rne(f4, f5), pack_bf16_rne(f6, f7)};
-        bf16x8 o;
-        __builtin_memcpy(&o, &r, 16);
-        return o;
-    }
 };
 
 struct FmtI8Row {
@@ -244,7 +225,7 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
             const u32x4 q = cq[nb];
             if constexpr (i4) {
                 const uint32_t wsel = t == 0 ? q.x : t == 1 ? q.y : t == 2 ? q.z : q.w;
-                bf[set][t][nb] = FmtI4G32::dequant(wsel, cs[nb][0], cs[nb][1], cs[nb][2], cs[nb][3], c_mlo, c_mhi, c_magic);
+                bf[set][t][nb] = dequant8_i4(wsel, cs[nb][0], cs[nb][1], cs[nb][2], cs[nb][3], c_mlo, c_mhi, c_magic);
             } else {
                 bf[set][t][nb] = t == 0 ? FmtI8Row::dequant(q.x, q.y) : FmtI8Row::dequant(q.z, q.w);
             }
@@ -442,8 +423,21 @@ static int launch_gemm(const uint16_t *x, const void *wq, const typename F::scal
     return launch_gemm_g<F, 2, false, OUTF32>(x, wq, sc, y, M, N, K, groups, ngroups, st);
 }
 
+bool gemm_big_i4g32_ok(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, int M, int N, int K);
+int gemm_big_i4g32_launch(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, uint16_t *y, int M, int N, int K, hipStream_t st);
+
 int gemm_i4g32_bf16_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, uint16_t *y, int M, int N,
                              int K, hipStream_t st) {
+    // many rows: the 256 x 256 tile, which dequantises a weight once per 256 rows, as soon as its tiles cover most of
+    // the chip (a tile alone on a compute unit takes about as long as all of them together: at 4096 columns the small
+    // tile is still ahead at 2048 rows, 101 against 115 us).  CHADQ_GEMM_TILE=big / small overrides the choice.
+    static const int force = [] {
+        const char *e = getenv("CHADQ_GEMM_TILE");
+        return !e ? 0 : (e[0] == 'b' ? 1 : (e[0] == 's' ? -1 : 0));
+    }();
+    const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+    if (force >= 0 && (force > 0 || big_tiles >= 176) && gemm_big_i4g32_ok(x, wp, sc, M, N, K))
+        return gemm_big_i4g32_launch(x, wp, sc, y, M, N, K, st);
     return launch_gemm<FmtI4G32, false>(x, wp, sc, y, M, N, K, nullptr, 0, st);
 }
 

@@ -21,27 +21,6 @@ namespace chadq {
 constexpr int SK_MT = 96;   // tokens per workgroup tile
 constexpr int SK_KI = 64;   // k per iteration
 
-struct SkDequant {
-    // 8 nibbles of word `w` -> 8 bf16 of (u-8)*s in k order; see FmtI4G32::dequant in the prefill kernel for the
-    // magic-number scheme (0x6400|u reads 1024+u, a nibble left in bits 7:4 reads 1024+16u).
-    __device__ static __forceinline__ bf16x8 run(uint32_t w, float s, float s16, float c0, float c1, uint32_t mlo,
-                                                 uint32_t mhi, uint32_t magic) {
-        const f16x2 h0 = as_f16x2(and_or(w, mlo, magic));
-        const f16x2 h1 = as_f16x2(and_or(w, mhi, magic));
-        const uint32_t w8 = w >> 8;
-        const f16x2 h2 = as_f16x2(and_or(w8, mlo, magic));
-        const f16x2 h3 = as_f16x2(and_or(w8, mhi, magic));
-        const float f0 = __builtin_fmaf((float)h0.x, s, c0), f4 = __builtin_fmaf((float)h0.y, s, c0);
-        const float f1 = __builtin_fmaf((float)h1.x, s16, c1), f5 = __builtin_fmaf((float)h1.y, s16, c1);
-        const float f2 = __builtin_fmaf((float)h2.x, s, c0), f6 = __builtin_fmaf((float)h2.y, s, c0);
-        const float f3 = __builtin_fmaf((float)h3.x, s16, c1), f7 = __builtin_fmaf((float)h3.y, s16, c1);
-        const u32x4 r = {pack_bf16_rne(f0, f1), pack_bf16_rne(f2, f3), pack_bf16_rne(f4, f5), pack_bf16_rne(f6, f7)};
-        bf16x8 o;
-        __builtin_memcpy(&o, &r, 16);
-        return o;
-    }
-};
-
 // Operand supply: everything comes global -> LDS by DMA, ahead of its use, so that memory latency is covered by
 // bytes in flight rather than by registers or occupancy:
 //   activation ring (shared by the workgroup): 3 stages of 32*SK_MB rows x 64 k, each wave fetches a quarter,
@@ -178,7 +157,7 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
         bf16x8 bf[2][2];
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb)
-            bf[0][nb] = SkDequant::run(q[nb].x, cs[nb][0], cs[nb][1], cs[nb][2], cs[nb][3], c_mlo, c_mhi, c_magic);
+            bf[0][nb] = dequant8_i4(q[nb].x, cs[nb][0], cs[nb][1], cs[nb][2], cs[nb][3], c_mlo, c_mhi, c_magic);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             if (j < 3) {
@@ -196,7 +175,7 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
 #pragma unroll
                 for (int nb = 0; nb < 2; ++nb) {
                     const uint32_t wsel = j == 0 ? q[nb].y : j == 1 ? q[nb].z : q[nb].w;
-                    bf[(j + 1) & 1][nb] = SkDequant::run(wsel, cs[nb][0], cs[nb][1], cs[nb][2], cs[nb][3], c_mlo, c_mhi, c_magic);
+                    bf[(j + 1) & 1][nb] = dequant8_i4(wsel, cs[nb][0], cs[nb][1], cs[nb][2], cs[nb][3], c_mlo, c_mhi, c_magic);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);

@@ -237,13 +237,6 @@ int chadq_argmax_f32(const float *v, int n, void *scratch, int32_t *token, int32
 int chadq_sample_topk_f32(const float *v, int n, int k, float temperature, const float *u, void *workspace, int32_t *token,
                           int32_t *pos, int advance, void *stream);
 
-/*
- * A measuring aid with no counterpart in any runtime: reads the first bytes / 16384 * 16384 bytes of src with the decode
- * GEMV's access shape and nothing else (four 1-KiB loads in flight per wave), and stores one word per 16 KiB to out
- * (bytes / 16384 words).  bench.py times it beside the GEMV to show what a cold read of the same size costs here.
- */
-int chadq_probe_read(const void *src, int64_t bytes, uint32_t *out, void *stream);
-
 #ifdef __cplusplus
 }
 #endif

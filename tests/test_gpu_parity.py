@@ -93,15 +93,21 @@ def test_dequant_exact(ops):
     assert np.array_equal(ops.dequantize(q8).cpu().numpy(), O.dequant_int8(w, s8))
 
 
-def test_probe_read_reads_every_byte(ops):
-    from chadslab_amd import _lib
+def test_bench_probe_reads_every_byte():
+    # the loads-only kernel bench.py times beside the GEMV lives in its own small library next to bench.py
+    import ctypes
 
-    lib = _lib.load()
+    path = os.path.join(os.path.dirname(GOLD.rstrip(os.sep)), os.pardir, "bench_probe.so")
+    if not os.path.exists(path):
+        pytest.skip("bench_probe.so has not been built (__graft_entry__.build() builds it)")
+    lib = ctypes.CDLL(os.path.abspath(path))
+    lib.bench_probe_read.restype = ctypes.c_int
+    lib.bench_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
     n = 5 * 16384 + 100  # the tail that does not fill 16 KiB is left alone
     data = rng(11).integers(0, 256, n, dtype=np.uint8)
     t = torch.from_numpy(data).to(DEV)
     out = torch.zeros(n // 16384, dtype=torch.int32, device=DEV)
-    _lib.check(lib.chadq_probe_read(t.data_ptr(), n, out.data_ptr(), torch.cuda.current_stream().cuda_stream), "probe")
+    assert lib.bench_probe_read(t.data_ptr(), n, out.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0
     want = np.bitwise_xor.reduce(data[:5 * 16384].view(np.uint32).reshape(5, -1), axis=1)
     assert np.array_equal(out.cpu().numpy().view(np.uint32), want)
 
@@ -289,6 +295,38 @@ def test_gemm_int8(ops, m, n, k):
     xb = O.f32_to_bf16(x)
     y = O.bf16_to_f32(bits(ops.qgemm(bf16_tensor(xb), q8)))
     assert O.rel_l2(y, O.qgemm_int8_f64(xb, w, s)) <= TOL_BF16
+
+
+@pytest.mark.parametrize("m,n,k", [(4096, 4096, 512), (3300, 3500, 256), (2817, 4099, 768), (8192, 1536, 1024)])
+def test_gemm_int4_many_rows_tile(ops, m, n, k):
+    # enough 256 x 256 tiles to cover the chip: these shapes run on the large-tile kernel (K a multiple of 256), with
+    # ragged last tiles in both directions and, for n = 4099, rows the vector stores cannot take
+    packed, s, xb, qw = i4_case(600 + m + n + k, m, n, k)
+    y = O.bf16_to_f32(bits(ops.qgemm(bf16_tensor(xb), qw)))
+    assert y.shape == (m, n) and np.isfinite(y).all()
+    assert O.rel_l2(y, O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_BF16
+
+
+def test_gemm_int4_many_rows_full_k_and_integer_exact(ops):
+    from chadslab_amd import QWeightInt4G32
+
+    # 4096 x 4096 x 4096: the float64 truth is formed for a sample of rows only (the oracle's full product would take
+    # minutes); every row of the result is still checked for being finite
+    m = n = k = 4096
+    packed, s, xb, qw = i4_case(611, m, n, k)
+    y = O.bf16_to_f32(bits(ops.qgemm(bf16_tensor(xb), qw)))
+    assert np.isfinite(y).all()
+    rows = rng(612).choice(m, 96, replace=False)
+    rows[:4] = (0, 255, 256, 4095)
+    assert O.rel_l2(y[rows], O.qgemm_int4g32_f64(xb[rows], packed, s)) <= TOL_BF16
+    # integer activations and unit scales: every sum is an integer below 2^24, so fp32 accumulation is exact and the
+    # only rounding is the final one to bf16
+    xi = O.f32_to_bf16(rng(613).integers(-4, 5, (m, 1024)).astype(np.float32))
+    pk, _, _, q1 = i4_case(614, 1, n, 1024)
+    yi = bits(ops.qgemm(bf16_tensor(xi), QWeightInt4G32(q1.packed, torch.ones_like(q1.scale))))
+    brute = O.bf16_to_f32(xi[rows]).astype(np.float64) @ O.unpack_int4(pk).astype(np.float64).T
+    assert np.abs(brute).max() < 2 ** 24
+    assert np.array_equal(yi[rows], O.f32_to_bf16(brute.astype(np.float32)))
 
 
 def test_gemm_agrees_with_gemv_at_m8(ops):
