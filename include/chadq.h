@@ -76,7 +76,8 @@ int chadq_dequant_i8row(const int8_t *w8, const float *scale, float *w, int N, i
 /*
  * y[m,n] = sum_g float(scale[n,g]) * sum_{k in g} x[m,k] * (u[n,k]-8)      (config 1)
  * x bf16 [M,K], y fp32 [M,N], 1 <= M <= 16, K % 32 == 0.  wp and x 16-byte aligned.
- * HBM-bound: each packed weight byte and each scale is read once for all M rows.
+ * HBM-bound: each packed weight byte and each scale is read once for up to 8 activation rows; 9 to 16 rows run as
+ * two launches of up to 8 rows each and stream the weights twice.
  */
 int chadq_gemv_i4g32(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *scale_f16, float *y, int M, int N,
                      int K, void *stream);
@@ -109,6 +110,9 @@ int chadq_gemv_i4g32_addnorm(const float *res, const float *delta, int n_delta, 
 /*
  * y[m,n] = scale[n] * sum_k x[m,k] * W[n,k]                                 (config 0)
  * x fp32 [M,K], W int8 [N,K], scale fp32 [N], y fp32 [M,N], 1 <= M <= 16, K % 16 == 0.
+ * The weights are streamed once per pair of activation rows (M = 1, 2: once; M = 16: eight times): the fp32
+ * activations leave registers for two rows' sums only.  Batched decode belongs on the int4 path or on
+ * chadq_gemm_i8row_bf16.
  */
 int chadq_gemv_i8row(const float *x, const int8_t *w8, const float *scale, float *y, int M, int N, int K,
                      void *stream);
@@ -158,7 +162,10 @@ int chadq_moe_ffn_i4g32(const uint16_t *x_bf16, const float *logits, const chadq
                         size_t workspace_bytes, void *stream);
 
 /* ---- decode-step pieces around the GEMVs (benchmark config 4), batch 1 ------------------- */
-/* The position and the current token live in device memory so that one captured HIP graph serves every step. */
+/* The position and the current token live in device memory so that one captured HIP graph serves every step.
+ * The kernels clamp pos[0] to [0, max_ctx-1] and token[0] to [0, V-1] so that nothing is addressed out of bounds, and
+ * report nothing when they do: a step past the end of the cache overwrites its last row and rotates by the wrong
+ * angle.  Keeping pos + steps <= max_ctx is the caller's job (QuantDecoder.feed / generate check it on the host). */
 
 /* x[d] fp32 = dequantised row token[0] (clamped to [0,V-1]) of the tied int4 group-32 table [V,d]. */
 int chadq_embed_i4g32(const int32_t *token, const uint8_t *wp, const uint16_t *scale_f16, float *x, int d, int V,
