@@ -21,7 +21,8 @@
 //   C = -136 * sum of the group's activations, which turns 128+u into u-8.  For integer-valued activations
 //       every term is an exact fp32 integer, so integer accumulation stays bit-exact.
 // HP trades activation rows per pass for contiguity of the weight stream: M = 1 runs HP = 4, M = 2 runs
-// HP = 2, M >= 3 runs HP = 1 (two passes over the same unpacked weights for M > 4).
+// HP = 2, M = 3 and 4 run HP = 1.  Five to eight rows run gemv_i4g32_mfma_pair_kernel further down, which
+// regroups the loaded words between lane groups so that eight rows fit one pass.
 //
 // Workgroup = 4*RBW waves; each group of 4 waves covers 16 weight rows.  K is consumed in chunks of 4096;
 // a wave takes 8 steps of a chunk (8 x 16 B per lane in flight), so 4/HP waves split a chunk of one row
@@ -65,8 +66,7 @@ struct GemvCfg {
     static constexpr int XI = (MPASS * (KC / 8) + T - 1) / T;  // 16-byte activation pieces per thread per pass
 };
 
-// waves_per_eu(4): at most 128 VGPRs, which also makes the compiler pick the MFMA form that writes VGPRs.  The
-// variants for 5 to 8 activation rows with 16 steps per wave need a few more (they spilled at 128): 3 waves, 168.
+// waves_per_eu(4): at most 128 VGPRs, which also makes the compiler pick the MFMA form that writes VGPRs.
 // XM: how the activation vector comes about (M = 1 for the modes other than 0).
 //   0  given: x bf16 [M,K].
 //   1  GeGLU folded in: x[k] = bf16( gelu_tanh(gu[k]) * gu[K + k] ) from gu fp32 [2K] (`x` points at gu) - a gated FFN's
@@ -82,7 +82,7 @@ struct GemvPre {
 };
 
 template <int MT, int HP, int S, int RBW, int D, int KC, int XM = 0>
-__global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((MT >= 5 && S == 16) ? 3 : 4))) void gemv_i4g32_mfma_kernel(
+__global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) void gemv_i4g32_mfma_kernel(
     const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
     float *__restrict__ y, int N, int K, int kspan, int pv, GemvPre pre) {
     constexpr bool XG = (XM == 1), XN = (XM == 2);
@@ -343,6 +343,221 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((MT >
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Eight rows of A per scale group: up to 8 activation rows with one K-part, up to 4 with two.
+//
+// The kernel above gives every lane group j of an MFMA column its own scale group, which leaves four rows of A per
+// group.  Here the two lane-group pairs (0,1) and (2,3) each work on one scale group, eight rows of A per group:
+//   load     as above: lane (n = h*P + r, j) fetches the 16 bytes of group (c*HP + h)*4 + j of weight row r.
+//   exchange v_permlane16_swap on words (0,1) and on words (2,3): lane groups 0 and 1 then hold group 4(c*HP+h)
+//            (pair 0) and the next one (pair 1), lane groups 2 and 3 the two after those - word `half` of each, lane
+//            group j & 1 supplying k 16*half + 8*(j&1) .. +7 of the group.  Two instructions per 16-byte load.
+//   A        row i = 8*g + v (g = which of the pair's two groups, v = h'*MR + m, MR = 8/HP activation rows); real
+//            data where the lane's k-slot group j has j >> 1 == g, zeros elsewhere.
+//   D        lane (n, j) holds rows 8*(j>>1) + 4*(j&1) .. +3 of its column: one scale per lane and pair, four FMAs;
+//            meaningful where the row's K-part h' equals the column's h.
+// Per 16-byte load: 4 MFMAs and 8 scale FMAs.  With HP = 1 that serves 5 to 8 activation rows in one pass (the form
+// above would need 8 and 8): 9.4-9.6 us against 10.4-10.7 at 14336 x 4096 and 8 rows.  HP = 2 would give 3 and 4 rows
+// the load shape of a single row (8 weight rows x 128 contiguous bytes per instruction instead of 16 x 64); it is
+// correct but measured slower than the form above there (8.6 against 8.2 us), so only HP = 1 is dispatched.
+template <int HP, int S, int RBW, int KC>
+struct GemvPairCfg {
+    static constexpr int P = 16 / HP;
+    static constexpr int MR = 8 / HP;
+    static constexpr int STEPS = KC / (128 * HP);
+    static constexpr int KS = STEPS / S;
+    static constexpr int UR = P * 4 / KS;
+    static_assert(HP == 1 || HP == 2, "one or two K-parts");
+    static_assert(KS >= 1 && KS <= 4 && KS * S == STEPS, "a chunk of one row block is split over 1, 2 or 4 waves");
+    static constexpr int XA_BYTES = STEPS * 2048;  // A operands: [c][pair][half][g][j&1][v] x 16 B
+    static constexpr int NX_BYTES = STEPS * 128;   // C operands: [c][pair][j][v%4] fp32
+    static constexpr int ZERO_OFF = XA_BYTES + NX_BYTES;
+    static constexpr int ZERO_SPAN = 2048;  // lanes off the diagonal add the same per-MFMA offsets (up to 1536) as the others
+    static constexpr int SC_OFF = ZERO_OFF + ZERO_SPAN;
+    static constexpr int SC_PPR = S * HP / 2;
+    static constexpr int SC_PITCH = SC_PPR * 16 + 16;
+    static constexpr int SC_NL = (P * SC_PPR + 63) / 64;
+    static constexpr int SC_WAVE = P * SC_PITCH;
+    static constexpr int OPER_BYTES = SC_OFF + RBW * 4 * SC_WAVE;
+    static constexpr int RED_BYTES = RBW * 4 * 64 * 16;
+    static constexpr int TOTAL = OPER_BYTES > RED_BYTES ? OPER_BYTES : RED_BYTES;
+    static constexpr int T = 256 * RBW;
+    static constexpr int XI = (MR * (KC / 8) + T - 1) / T;  // 16-byte activation pieces per thread and chunk
+    static_assert((MR * (KC / 8)) % T == 0, "whole rounds of pieces");
+};
+
+template <int MT, int HP, int S, int RBW, int D, int KC>
+__global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((HP == 1 && S == 16) ? 2 : 4))) void gemv_i4g32_mfma_pair_kernel(
+    const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
+    float *__restrict__ y, int N, int K, int pv) {
+    typedef GemvPairCfg<HP, S, RBW, KC> C;
+    constexpr int M = MT, P = C::P, MR = C::MR, KS = C::KS, T = C::T, XI = C::XI;
+    static_assert(M >= 1 && M <= MR, "eight rows of A per scale group, shared by the K-parts");
+    // HP = 1, S = 16: one 8-wave workgroup per compute unit (its LDS), so a wave may use 256 registers
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int unit = wave >> 2, wv = wave & 3;
+    const int rbs = wv / KS, ks = wv % KS;
+    const int nl = lane & 15, j = lane >> 4;
+    const int h = nl / P, r = nl % P;
+    const int n0 = ((blockIdx.x * RBW + unit) * (4 / KS) + rbs) * pv;
+    const int KH = K >> 1, G = K >> 5;
+    const int row = (r < pv && n0 + r < N) ? n0 + r : (n0 < N ? n0 : N - 1);
+    const uint32_t wrow = (uint32_t)row * (uint32_t)KH;
+    const uint32_t mask_r = vgpr_const(0x000F000Fu), magic_r = vgpr_const(kBf16Magic);
+
+    for (int o = tid * 16; o < C::ZERO_SPAN; o += T * 16) *reinterpret_cast<u32x4 *>(lds + C::ZERO_OFF + o) = u32x4{0, 0, 0, 0};
+
+    // A operand: lane (i = lane & 15, j) is row 8g + v with g = i >> 3, v = i & 7 = h'*MR + m
+    const bool a_live = ((nl >> 3) == (j >> 1)) && (((nl & 7) % MR) < M);
+    const uint32_t a_base = a_live ? (uint32_t)(ks * S * 2048 + (j >> 1) * 256 + (j & 1) * 128 + (nl & 7) * 16) : (uint32_t)C::ZERO_OFF;
+    const uint32_t a_step = a_live ? 2048u : 0u;
+
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    uint8_t *sct = lds + C::SC_OFF + wave * C::SC_WAVE;
+    int srow_l[C::SC_NL], spiece[C::SC_NL], srow[C::SC_NL];
+#pragma unroll
+    for (int l = 0; l < C::SC_NL; ++l) {
+        srow_l[l] = (lane + 64 * l) / C::SC_PPR;
+        spiece[l] = (lane + 64 * l) % C::SC_PPR;
+        srow[l] = (srow_l[l] < pv && n0 + srow_l[l] < N) ? n0 + srow_l[l] : (n0 < N ? n0 : N - 1);
+    }
+
+    // Piece it = tid + T*q of a chunk: word t = it % 4 of its scale group (the four pieces of a group in one quad of
+    // lanes), activation row m = it / 4 % MR, then K-part hh, pair, g and step from the bits above.  A wave's store
+    // to LDS is four runs of 256 contiguous bytes (conflict free), its load runs of 128 contiguous bytes per row.
+    auto piece = [&](int it, int &t, int &m, int &c, int &hh, int &pr, int &g) {
+        t = it & 3;
+        m = (it >> 2) % MR;
+        int rest = (it >> 2) / MR;
+        hh = rest % HP;
+        rest /= HP;
+        pr = rest & 1;
+        g = (rest >> 1) & 1;
+        c = rest >> 2;
+    };
+
+    for (int kc0 = 0; kc0 < K; kc0 += KC) {
+        // 1. activation loads first
+        u32x4 xr[XI];
+#pragma unroll
+        for (int q = 0; q < XI; ++q) {
+            int t, m, c, hh, pr, g;
+            piece(tid + T * q, t, m, c, hh, pr, g);
+            const int k = kc0 + 32 * ((c * HP + hh) * 4 + g * 2 + pr) + 8 * t;
+            xr[q] = u32x4{0, 0, 0, 0};
+            if (m < M && k < K) xr[q] = *reinterpret_cast<const u32x4 *>(x + (size_t)m * K + k);
+        }
+        // 2. the wave's scale tile
+        u32x4 sv[C::SC_NL];
+#pragma unroll
+        for (int l = 0; l < C::SC_NL; ++l) {
+            const int gs = (kc0 >> 5) + ks * S * 4 * HP + spiece[l] * 8;
+            sv[l] = *reinterpret_cast<const u32x4 *>(sc + ((size_t)srow[l] * G + (gs < G ? gs : 0)));
+            if (gs >= G) sv[l] = u32x4{0, 0, 0, 0};
+        }
+        // 3. the first D weight loads
+        u32x4 w[S];
+        auto issue_w = [&](int i) {
+            const int gg = (kc0 >> 5) + ((S * ks + i) * HP + h) * 4 + j;
+            w[i] = load_nt_b128(wp + (wrow + (uint32_t)(gg < G ? gg : 0) * 16u));
+        };
+#pragma unroll
+        for (int i = 0; i < (D < S ? D : S); ++i) issue_w(i);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // 4. stage the activations
+        __syncthreads();  // the previous chunk's operand reads (or the zero fill) are done
+#pragma unroll
+        for (int l = 0; l < C::SC_NL; ++l)
+            if (srow_l[l] < P) *reinterpret_cast<u32x4 *>(sct + srow_l[l] * C::SC_PITCH + spiece[l] * 16) = sv[l];
+#pragma unroll
+        for (int q = 0; q < XI; ++q) {
+            int t, m, c, hh, pr, g;
+            piece(tid + T * q, t, m, c, hh, pr, g);
+            uint32_t a[4] = {xr[q].x, xr[q].y, xr[q].z, xr[q].w}, o[4];
+            float sum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum = dot2_bf16(a[e], 0x3F803F80u, sum);
+            pair_x8(a, o);
+            const int v = hh * MR + m;
+            if (m < M)
+                *reinterpret_cast<u32x4 *>(lds + c * 2048 + (pr * 2 + (t >> 1)) * 512 + g * 256 + (t & 1) * 128 + v * 16) =
+                    u32x4{o[0], o[1], o[2], o[3]};
+            sum += dpp_f32<0xB1, 0xF>(sum);  // the four pieces of a group sit in four adjacent lanes
+            sum += dpp_f32<0x4E, 0xF>(sum);
+            if (t == 0 && m < M)
+                *reinterpret_cast<float *>(lds + C::XA_BYTES + ((c * 2 + pr) * 4 + g * 2 + (v >> 2)) * 16 + (v & 3) * 4) =
+                    -kMagicBias * sum;
+        }
+        __syncthreads();
+
+        // 5. the chunk's S steps of this wave
+        uint32_t a_addr = a_base;
+#pragma unroll
+        for (int i = 0; i < S; ++i) {
+            const int c = S * ks + i;
+            if (D < S) {
+                asm volatile("" : "+v"(w[i]));
+                if (i + D < S) issue_w(i + D);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            const u32x2 lo = __builtin_amdgcn_permlane16_swap(w[i].x, w[i].y, false, false);
+            const u32x2 hi = __builtin_amdgcn_permlane16_swap(w[i].z, w[i].w, false, false);
+            uint32_t pw[16];  // [pair][half][4]
+            unpack8_magic_r(lo.x, mask_r, magic_r, &pw[0]);
+            unpack8_magic_r(hi.x, mask_r, magic_r, &pw[4]);
+            unpack8_magic_r(lo.y, mask_r, magic_r, &pw[8]);
+            unpack8_magic_r(hi.y, mask_r, magic_r, &pw[12]);
+#pragma unroll
+            for (int pr = 0; pr < 2; ++pr) {
+                const float s = f16_bits_to_f32(
+                    *reinterpret_cast<const uint16_t *>(sct + r * C::SC_PITCH + ((i * HP + h) * 4 + pr + 2 * (j >> 1)) * 2));
+                f32x4 d = *reinterpret_cast<const f32x4 *>(lds + C::XA_BYTES + ((2 * c + pr) * 4 + j) * 16);
+#pragma unroll
+                for (int hf = 0; hf < 2; ++hf) {
+                    const bf16x8 av = *reinterpret_cast<const bf16x8 *>(lds + a_addr + (pr * 2 + hf) * 512);
+                    const u32x4 bw = {pw[(pr * 2 + hf) * 4], pw[(pr * 2 + hf) * 4 + 1], pw[(pr * 2 + hf) * 4 + 2], pw[(pr * 2 + hf) * 4 + 3]};
+                    bf16x8 bv;
+                    __builtin_memcpy(&bv, &bw, 16);
+                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, d, 0, 0, 0);
+                }
+                acc += d * s;
+            }
+            a_addr += a_step;
+        }
+    }
+
+    // 6. fold the two scale-group halves, the K-parts and the K-slices
+    __syncthreads();
+    u32x4 *red = reinterpret_cast<u32x4 *>(lds);
+    {
+        u32x4 v;
+        __builtin_memcpy(&v, &acc, 16);
+        red[wave * 64 + lane] = v;
+    }
+    __syncthreads();
+    constexpr int UR = C::UR, OUT_PER_UNIT = UR * MR;
+    for (int o = tid; o < RBW * OUT_PER_UNIT; o += T) {
+        const int n16 = o % UR, m = (o / UR) % MR, un = o / OUT_PER_UNIT;
+        const int rb = n16 / P, rr = n16 % P;
+        float t = 0.f;
+#pragma unroll
+        for (int k4 = 0; k4 < KS; ++k4)
+#pragma unroll
+            for (int hh = 0; hh < HP; ++hh)
+#pragma unroll
+                for (int g = 0; g < 2; ++g) {
+                    const int v = hh * MR + m;
+                    const int wsrc = un * 4 + rb * KS + k4, lsrc = 16 * (2 * g + (v >> 2)) + hh * P + rr;
+                    t += reinterpret_cast<const float *>(red)[(wsrc * 64 + lsrc) * 4 + (v & 3)];
+                }
+        const int nn = ((blockIdx.x * RBW + un) * (4 / KS) + rb) * pv + rr;
+        if (rr < pv && nn < N && m < M) y[(size_t)m * N + nn] = t;
+    }
+}
+
 int gemv_i4g32_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
 
 // Rows of a P-row tile to use.  All workgroups of these grids are resident at once, so the launch lasts as long as
@@ -393,6 +608,23 @@ static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc,
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma launch");
 }
 
+template <int MT, int HP, int S, int RBW, int D, int KC = 4096>
+static int launch_pair(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K, hipStream_t st) {
+    typedef GemvPairCfg<HP, S, RBW, KC> C;
+    static std::atomic<bool> attr_set{false};
+    if (!attr_set.load(std::memory_order_acquire)) {
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_pair_kernel<MT, HP, S, RBW, D, KC>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, C::TOTAL));
+        attr_set.store(true, std::memory_order_release);
+    }
+    const int tiles_per_wg = 4 / C::KS * RBW;
+    const int pv = pick_tile_rows(N, C::P, tiles_per_wg, 1);
+    const int tiles = (N + pv - 1) / pv;
+    hipLaunchKernelGGL((gemv_i4g32_mfma_pair_kernel<MT, HP, S, RBW, D, KC>), dim3((tiles + tiles_per_wg - 1) / tiles_per_wg), dim3(256 * RBW),
+                       C::TOTAL, st, x, wp, sc, y, N, K, pv);
+    return hip_check(hipGetLastError(), "gemv_i4g32_mfma_pair launch");
+}
+
 int gemv_i4g32_mfma_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int M, int N, int K,
                              hipStream_t st) {
     // the matrix-core kernel wants 16-byte aligned scale rows (K % 256 == 0) and 32-bit byte offsets
@@ -427,16 +659,16 @@ int gemv_i4g32_mfma_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_
                 rc = tall ? launch_mfma<4, 1, 16, 1, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<4, 1, 8, 1, 8>(xm, wp, sc, ym, N, K, st);
                 break;
             case 5:
-                rc = tall ? launch_mfma<5, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<5, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
+                rc = tall ? launch_pair<5, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_pair<5, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
                 break;
             case 6:
-                rc = tall ? launch_mfma<6, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<6, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
+                rc = tall ? launch_pair<6, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_pair<6, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
                 break;
             case 7:
-                rc = tall ? launch_mfma<7, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<7, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
+                rc = tall ? launch_pair<7, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_pair<7, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
                 break;
             default:
-                rc = tall ? launch_mfma<8, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<8, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
+                rc = tall ? launch_pair<8, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_pair<8, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
                 break;
         }
         if (rc != 0) return rc;
