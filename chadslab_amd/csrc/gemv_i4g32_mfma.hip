@@ -558,6 +558,182 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((HP =
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Sixteen rows of A per scale group: 9 to 16 activation rows in one pass over the weights.
+//
+// After v_permlane16_swap on words (0,1) and (2,3) as above, v_permlane32_swap between the two results moves the
+// halves of a group together: register t of a lane then holds word j (= the lane's group of 16 lanes) of scale
+// group 4c + t, so MFMA t works on ONE scale group with all four k-slot groups and all 16 rows of A are activation
+// rows.  Per 16-byte load: 4 exchanges, 4 MFMAs, 16 scale FMAs.  M is a run-time argument (rows past M read zeros).
+template <int S, int RBW, int KC>
+struct GemvRows16Cfg {
+    static constexpr int P = 16;
+    static constexpr int STEPS = KC / 128;
+    static constexpr int KS = STEPS / S;
+    static constexpr int UR = P * 4 / KS;
+    static_assert(KS >= 1 && KS <= 4 && KS * S == STEPS, "a chunk of one row block is split over 1, 2 or 4 waves");
+    static constexpr int XA_BYTES = STEPS * 4096;  // A operands: [c][t][word j][row i] x 16 B
+    static constexpr int NX_BYTES = STEPS * 256;   // C operands: [c][t][j][v] fp32
+    static constexpr int ZERO_OFF = XA_BYTES + NX_BYTES;
+    static constexpr int ZERO_SPAN = 4096;         // rows past M add the same per-MFMA offsets (up to 3072) as the others
+    static constexpr int SC_OFF = ZERO_OFF + ZERO_SPAN;
+    static constexpr int SC_PPR = S / 2;
+    static constexpr int SC_PITCH = SC_PPR * 16 + 16;
+    static constexpr int SC_NL = (P * SC_PPR + 63) / 64;
+    static constexpr int SC_WAVE = P * SC_PITCH;
+    static constexpr int OPER_BYTES = SC_OFF + RBW * 4 * SC_WAVE;
+    static constexpr int RED_BYTES = RBW * 4 * 64 * 16;
+    static constexpr int TOTAL = OPER_BYTES > RED_BYTES ? OPER_BYTES : RED_BYTES;
+    static constexpr int T = 256 * RBW;
+    static constexpr int XI = (16 * (KC / 8)) / T;  // 16-byte activation pieces per thread and chunk
+    static_assert((16 * (KC / 8)) % T == 0, "whole rounds of pieces");
+};
+
+template <int S, int RBW, int D, int KC>
+__global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(RBW == 2 ? 2 : 4))) void gemv_i4g32_mfma_rows16_kernel(
+    const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
+    float *__restrict__ y, int M, int N, int K, int pv) {
+    typedef GemvRows16Cfg<S, RBW, KC> C;
+    constexpr int P = C::P, KS = C::KS, T = C::T, XI = C::XI;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int unit = wave >> 2, wv = wave & 3;
+    const int rbs = wv / KS, ks = wv % KS;
+    const int r = lane & 15, j = lane >> 4;
+    const int n0 = ((blockIdx.x * RBW + unit) * (4 / KS) + rbs) * pv;
+    const int KH = K >> 1, G = K >> 5;
+    const int row = (r < pv && n0 + r < N) ? n0 + r : (n0 < N ? n0 : N - 1);
+    const uint32_t wrow = (uint32_t)row * (uint32_t)KH;
+    const uint32_t mask_r = vgpr_const(0x000F000Fu), magic_r = vgpr_const(kBf16Magic);
+
+    for (int o = tid * 16; o < C::ZERO_SPAN; o += T * 16) *reinterpret_cast<u32x4 *>(lds + C::ZERO_OFF + o) = u32x4{0, 0, 0, 0};
+
+    const bool a_live = r < M;  // A row i = lane & 15 is activation row i
+    const uint32_t a_base = a_live ? (uint32_t)(ks * S * 4096 + j * 256 + r * 16) : (uint32_t)C::ZERO_OFF;
+    const uint32_t a_step = a_live ? 4096u : 0u;
+
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    uint8_t *sct = lds + C::SC_OFF + wave * C::SC_WAVE;
+    int srow_l[C::SC_NL], spiece[C::SC_NL], srow[C::SC_NL];
+#pragma unroll
+    for (int l = 0; l < C::SC_NL; ++l) {
+        srow_l[l] = (lane + 64 * l) / C::SC_PPR;
+        spiece[l] = (lane + 64 * l) % C::SC_PPR;
+        srow[l] = (srow_l[l] < pv && n0 + srow_l[l] < N) ? n0 + srow_l[l] : (n0 < N ? n0 : N - 1);
+    }
+
+    for (int kc0 = 0; kc0 < K; kc0 += KC) {
+        // 1. activation loads first.  Piece it = tid + T*q: word it % 4 of its scale group, activation row
+        //    it / 4 % 16, chunk-local group it / 64: a wave stores 1 KiB of contiguous LDS.
+        u32x4 xr[XI];
+#pragma unroll
+        for (int q = 0; q < XI; ++q) {
+            const int it = tid + T * q, m = (it >> 2) & 15, k = kc0 + 32 * (it >> 6) + 8 * (it & 3);
+            xr[q] = u32x4{0, 0, 0, 0};
+            if (m < M && k < K) xr[q] = *reinterpret_cast<const u32x4 *>(x + (size_t)m * K + k);
+        }
+        // 2. the wave's scale tile
+        u32x4 sv[C::SC_NL];
+#pragma unroll
+        for (int l = 0; l < C::SC_NL; ++l) {
+            const int gs = (kc0 >> 5) + ks * S * 4 + spiece[l] * 8;
+            sv[l] = *reinterpret_cast<const u32x4 *>(sc + ((size_t)srow[l] * G + (gs < G ? gs : 0)));
+            if (gs >= G) sv[l] = u32x4{0, 0, 0, 0};
+        }
+        // 3. the first D weight loads
+        u32x4 w[S];
+        auto issue_w = [&](int i) {
+            const int gg = (kc0 >> 5) + (S * ks + i) * 4 + j;
+            w[i] = load_nt_b128(wp + (wrow + (uint32_t)(gg < G ? gg : 0) * 16u));
+        };
+#pragma unroll
+        for (int i = 0; i < (D < S ? D : S); ++i) issue_w(i);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // 4. stage the activations
+        __syncthreads();  // the previous chunk's operand reads (or the zero fill) are done
+#pragma unroll
+        for (int l = 0; l < C::SC_NL; ++l)
+            if (srow_l[l] < P) *reinterpret_cast<u32x4 *>(sct + srow_l[l] * C::SC_PITCH + spiece[l] * 16) = sv[l];
+#pragma unroll
+        for (int q = 0; q < XI; ++q) {
+            const int it = tid + T * q, tw = it & 3, m = (it >> 2) & 15, gl = it >> 6;
+            const int c = gl >> 2, t = gl & 3;
+            uint32_t a[4] = {xr[q].x, xr[q].y, xr[q].z, xr[q].w}, o[4];
+            float sum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum = dot2_bf16(a[e], 0x3F803F80u, sum);
+            pair_x8(a, o);
+            if (m < M) *reinterpret_cast<u32x4 *>(lds + c * 4096 + t * 1024 + tw * 256 + m * 16) = u32x4{o[0], o[1], o[2], o[3]};
+            sum += dpp_f32<0xB1, 0xF>(sum);  // the four pieces of a group sit in four adjacent lanes
+            sum += dpp_f32<0x4E, 0xF>(sum);
+            if (tw == 0)  // rows past M get a zero correction
+                *reinterpret_cast<float *>(lds + C::XA_BYTES + ((c * 4 + t) * 4 + (m >> 2)) * 16 + (m & 3) * 4) =
+                    m < M ? -kMagicBias * sum : 0.f;
+        }
+        __syncthreads();
+
+        // 5. the chunk's S steps of this wave
+        uint32_t a_addr = a_base;
+#pragma unroll
+        for (int i = 0; i < S; ++i) {
+            const int c = S * ks + i;
+            if (D < S) {
+                asm volatile("" : "+v"(w[i]));
+                if (i + D < S) issue_w(i + D);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            const u32x2 lo = __builtin_amdgcn_permlane16_swap(w[i].x, w[i].y, false, false);
+            const u32x2 hi = __builtin_amdgcn_permlane16_swap(w[i].z, w[i].w, false, false);
+            const u32x2 g02 = __builtin_amdgcn_permlane32_swap(lo.x, hi.x, false, false);  // groups 4c and 4c+2
+            const u32x2 g13 = __builtin_amdgcn_permlane32_swap(lo.y, hi.y, false, false);  // groups 4c+1 and 4c+3
+            uint32_t pw[16];  // [t][4]
+            unpack8_magic_r(g02.x, mask_r, magic_r, &pw[0]);
+            unpack8_magic_r(g13.x, mask_r, magic_r, &pw[4]);
+            unpack8_magic_r(g02.y, mask_r, magic_r, &pw[8]);
+            unpack8_magic_r(g13.y, mask_r, magic_r, &pw[12]);
+            const u32x2 s4 = *reinterpret_cast<const u32x2 *>(sct + r * C::SC_PITCH + i * 8);  // the step's four scales
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint32_t sw = t < 2 ? s4.x : s4.y;
+                const float s = f16_bits_to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xFFFFu)));
+                f32x4 d = *reinterpret_cast<const f32x4 *>(lds + C::XA_BYTES + ((4 * c + t) * 4 + j) * 16);
+                const bf16x8 av = *reinterpret_cast<const bf16x8 *>(lds + a_addr + t * 1024);
+                const u32x4 bw = {pw[t * 4], pw[t * 4 + 1], pw[t * 4 + 2], pw[t * 4 + 3]};
+                bf16x8 bv;
+                __builtin_memcpy(&bv, &bw, 16);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, d, 0, 0, 0);
+                acc += d * s;
+            }
+            a_addr += a_step;
+        }
+    }
+
+    // 6. fold the K-slices
+    __syncthreads();
+    u32x4 *red = reinterpret_cast<u32x4 *>(lds);
+    {
+        u32x4 v;
+        __builtin_memcpy(&v, &acc, 16);
+        red[wave * 64 + lane] = v;
+    }
+    __syncthreads();
+    constexpr int UR = C::UR, OUT_PER_UNIT = UR * 16;
+    for (int o = tid; o < RBW * OUT_PER_UNIT; o += T) {
+        const int n16 = o % UR, m = (o / UR) % 16, un = o / OUT_PER_UNIT;
+        const int rb = n16 / P, rr = n16 % P;
+        float t = 0.f;
+#pragma unroll
+        for (int k4 = 0; k4 < KS; ++k4) {
+            const int wsrc = un * 4 + rb * KS + k4, lsrc = 16 * (m >> 2) + rr;
+            t += reinterpret_cast<const float *>(red)[(wsrc * 64 + lsrc) * 4 + (m & 3)];
+        }
+        const int nn = ((blockIdx.x * RBW + un) * (4 / KS) + rb) * pv + rr;
+        if (rr < pv && nn < N && m < M) y[(size_t)m * N + nn] = t;
+    }
+}
+
 int gemv_i4g32_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
 
 // Rows of a P-row tile to use.  All workgroups of these grids are resident at once, so the launch lasts as long as
@@ -625,12 +801,32 @@ static int launch_pair(const uint16_t *x, const uint8_t *wp, const uint16_t *sc,
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma_pair launch");
 }
 
+template <int S, int RBW, int D, int KC = 2048>
+static int launch_rows16(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int M, int N, int K, hipStream_t st) {
+    typedef GemvRows16Cfg<S, RBW, KC> C;
+    static std::atomic<bool> attr_set{false};
+    if (!attr_set.load(std::memory_order_acquire)) {
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_rows16_kernel<S, RBW, D, KC>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, C::TOTAL));
+        attr_set.store(true, std::memory_order_release);
+    }
+    const int tiles_per_wg = 4 / C::KS * RBW;
+    const int pv = pick_tile_rows(N, C::P, tiles_per_wg, 1);
+    const int tiles = (N + pv - 1) / pv;
+    hipLaunchKernelGGL((gemv_i4g32_mfma_rows16_kernel<S, RBW, D, KC>), dim3((tiles + tiles_per_wg - 1) / tiles_per_wg), dim3(256 * RBW),
+                       C::TOTAL, st, x, wp, sc, y, M, N, K, pv);
+    return hip_check(hipGetLastError(), "gemv_i4g32_mfma_rows16 launch");
+}
+
 int gemv_i4g32_mfma_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int M, int N, int K,
                              hipStream_t st) {
     // the matrix-core kernel wants 16-byte aligned scale rows (K % 256 == 0) and 32-bit byte offsets
     if ((K & 255) != 0 || (int64_t)N * (K / 2) >= ((int64_t)1 << 31) || (reinterpret_cast<uintptr_t>(sc) & 15u) != 0)
         return gemv_i4g32_dispatch(x, wp, sc, y, M, N, K, st);
-    // up to 8 activation rows per launch; more rows reuse the kernel on the next 8
+    // 9 to 16 activation rows: the 16-row form reads the weights once
+    if (M > 8 && M <= 16)
+        return N >= 8192 ? launch_rows16<8, 2, 4>(x, wp, sc, y, M, N, K, st) : launch_rows16<4, 1, 4>(x, wp, sc, y, M, N, K, st);
+    // up to 8 activation rows per launch (more than 16 rows: the kernels run on 8 rows at a time)
     for (int m0 = 0; m0 < M; m0 += 8) {
         const int mm = (M - m0) < 8 ? (M - m0) : 8;
         const uint16_t *xm = x + (size_t)m0 * K;

@@ -76,8 +76,8 @@ int chadq_dequant_i8row(const int8_t *w8, const float *scale, float *w, int N, i
 /*
  * y[m,n] = sum_g float(scale[n,g]) * sum_{k in g} x[m,k] * (u[n,k]-8)      (config 1)
  * x bf16 [M,K], y fp32 [M,N], 1 <= M <= 16, K % 32 == 0.  wp and x 16-byte aligned.
- * HBM-bound: each packed weight byte and each scale is read once for up to 8 activation rows; 9 to 16 rows run as
- * two launches of up to 8 rows each and stream the weights twice.
+ * HBM-bound: each packed weight byte and each scale is read once for all M <= 16 activation rows (the matrix-core
+ * kernels; the fallback for K % 256 != 0 or unaligned scales reads them once per pair of rows).
  */
 int chadq_gemv_i4g32(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *scale_f16, float *y, int M, int N,
                      int K, void *stream);

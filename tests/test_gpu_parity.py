@@ -144,7 +144,7 @@ def test_gemv_int4_shapes(ops, m, n, k):
     assert O.rel_l2(y, O.qgemm_int4g32_f64(xb, packed, s)) <= TOL_F32
 
 
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8, 13])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8, 9, 13, 16])
 def test_gemv_int4_config1_full_size(ops, m):
     packed, s, xb, qw = i4_case(1001, m, 14336, 4096)
     y = ops.qgemv(bf16_tensor(xb), qw).cpu().numpy()
@@ -181,7 +181,9 @@ def test_gemv_int4_output_table_256000_rows(ops, m):
     assert np.abs(brute).max() < 2 ** 24 and np.array_equal(yi, brute.astype(np.float32))
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 14336, 4096), (2, 14336, 4096), (8, 512, 4096), (4, 96, 256), (2, 40, 96)])
+@pytest.mark.parametrize("m,n,k", [(1, 14336, 4096), (2, 14336, 4096), (8, 512, 4096), (4, 96, 256), (2, 40, 96),
+                                   (5, 14336, 4096), (8, 14336, 4096), (6, 300, 512), (7, 8192, 256),
+                                   (9, 8192, 2048), (12, 14336, 4096), (16, 512, 4096), (16, 300, 512), (11, 64, 256)])
 def test_gemv_int4_integer_accumulation_bit_exact(ops, m, n, k):
     from chadslab_amd import QWeightInt4G32
 
