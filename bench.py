@@ -276,24 +276,40 @@ def main():
         x3 = torch.randn(T3, H3, device=dev, generator=g3).to(torch.bfloat16)
         z3 = torch.randn(T3, E3, device=dev, generator=g3)
         torch.cuda.synchronize()  # the inputs were generated on the default stream
-        with torch.cuda.stream(stream):
-            for _ in range(3):
-                ops.moe_ffn(x3, z3, experts)
-            a3, b3 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a3.record(stream)
-            for _ in range(n_moe):
-                ops.moe_ffn(x3, z3, experts)
-            b3.record(stream)
-            torch.cuda.synchronize()
-        us3 = a3.elapsed_time(b3) * 1000.0 / n_moe
+
+        def time_moe(ex):
+            with torch.cuda.stream(stream):
+                for _ in range(3):
+                    ops.moe_ffn(x3, z3, ex)
+                a3, b3 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a3.record(stream)
+                for _ in range(n_moe):
+                    ops.moe_ffn(x3, z3, ex)
+                b3.record(stream)
+                torch.cuda.synchronize()
+            return a3.elapsed_time(b3) * 1000.0 / n_moe
+
         hit = int(torch.unique(ops.moe_route(z3, 2, True)[0]).numel())
         flop3 = 2.0 * T3 * 2 * 3 * H3 * F3
         bytes3 = hit * 3 * (F3 * H3 // 2 + F3 * (H3 // 32) * 2)
-        extras["moe_ffn_i4g32_config3"] = {"us": round(us3, 1), "TFLOPs": round(flop3 / us3 * 1e-6, 1),
-                                           "frac_bf16_mfma_peak": round(flop3 / us3 * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4),
-                                           "experts_hit": hit, "expert_weight_GBps": round(bytes3 / us3 * 1e-3, 1),
-                                           "frac_hbm_peak": round(bytes3 / us3 * 1e-3 / HBM_PEAK_GBS, 4)}
-        del experts, x3, z3
+
+        def moe_entry(us3, note):
+            return {"us": round(us3, 1), "TFLOPs": round(flop3 / us3 * 1e-6, 1),
+                    "frac_bf16_mfma_peak": round(flop3 / us3 * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4), "experts_hit": hit,
+                    "expert_weight_GBps": round(bytes3 / us3 * 1e-3, 1),
+                    "frac_hbm_peak": round(bytes3 / us3 * 1e-3 / HBM_PEAK_GBS, 4), "weights": note}
+
+        extras["moe_ffn_i4g32_config3"] = moe_entry(time_moe(experts), "row-major containers")
+        # the same experts repacked once into tile order (ops.to_tiles, a load-time step outside the timed region)
+        with torch.cuda.stream(stream):
+            tiled = []
+            for tr in experts:  # one expert at a time: the row-major copy is dropped as soon as its tiles exist
+                tiled.append(tuple(ops.to_tiles(m) for m in tr))
+            torch.cuda.synchronize()
+        del experts
+        torch.cuda.empty_cache()
+        extras["moe_ffn_i4g32_config3_tiled"] = moe_entry(time_moe(tiled), "tile order (chadq_repack_i4g32_tiles at load time)")
+        del tiled, x3, z3
         torch.cuda.empty_cache()
     if "decode" in want:
         # config 4: decode step, 18 layers, d 2048, 8 query heads x 256, 1 KV head, FFN 16384, vocab 256000, batch 1,

@@ -54,7 +54,9 @@ int gemm_i8row_bf16_dispatch(const uint16_t *, const int8_t *, const float *, ui
 size_t moe_workspace_bytes(int, int, int, int, int);
 int moe_route_launch(const float *, int32_t *, float *, int, int, int, int, hipStream_t);
 int moe_ffn_i4g32_launch(const uint16_t *, const float *, const chadq_moe_expert_i4g32 *, uint16_t *, int, int, int, int, int,
-                         int, void *, hipStream_t);
+                         int, void *, bool, hipStream_t);
+bool moe_ffn_tiled_ok(int, int);
+int repack_i4g32_tiles_launch(const uint8_t *, const uint16_t *, uint8_t *, uint16_t *, int, int, bool, hipStream_t);
 
 int embed_launch(const int32_t *, const uint8_t *, const uint16_t *, float *, int, int, hipStream_t);
 int add_rmsnorm_launch(float *, const float *, int, const float *, uint16_t *, int, float, hipStream_t);
@@ -231,23 +233,62 @@ size_t chadq_moe_ffn_i4g32_workspace_bytes(int T, int H, int F, int E, int top_k
     return moe_workspace_bytes(T, H, F, E, top_k);
 }
 
+static int moe_ffn_entry(const char *name, bool tiled, const uint16_t *x_bf16, const float *logits,
+                         const chadq_moe_expert_i4g32 *experts, uint16_t *y_bf16, int T, int H, int F, int E, int top_k, int renorm,
+                         void *workspace, size_t workspace_bytes, hipStream_t st) {
+    CHADQ_REQUIRE(moe_sizes_ok(T, H, F, E, top_k), CHADQ_ERR_SHAPE,
+                  "%s: T=%d H=%d F=%d E=%d top_k=%d (H, F multiples of 32; E <= 16; top_k <= min(E, 8))", name, T, H, F, E, top_k);
+    CHADQ_REQUIRE(!tiled || moe_ffn_tiled_ok(H, F), CHADQ_ERR_SHAPE, "%s: H=%d and F=%d must be multiples of 256", name, H, F);
+    CHADQ_REQUIRE(x_bf16 && logits && experts && y_bf16, CHADQ_ERR_NULL, "%s: null pointer", name);
+    for (int e = 0; e < E; ++e)
+        CHADQ_REQUIRE(experts[e].wg && experts[e].sg && experts[e].wu && experts[e].su && experts[e].wd && experts[e].sd,
+                      CHADQ_ERR_NULL, "%s: expert %d has a null weight pointer", name, e);
+    const size_t need = moe_workspace_bytes(T, H, F, E, top_k);
+    CHADQ_REQUIRE(workspace && workspace_bytes >= need, CHADQ_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", name,
+                  need, workspace ? workspace_bytes : (size_t)0);
+    CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(workspace) && aligned16(y_bf16), CHADQ_ERR_ALIGN,
+                  "%s: x, y and workspace must be 16-byte aligned", name);
+    return moe_ffn_i4g32_launch(x_bf16, logits, experts, y_bf16, T, H, F, E, top_k, renorm, workspace, tiled, st);
+}
+
 int chadq_moe_ffn_i4g32(const uint16_t *x_bf16, const float *logits, const chadq_moe_expert_i4g32 *experts,
                         uint16_t *y_bf16, int T, int H, int F, int E, int top_k, int renorm, void *workspace,
                         size_t workspace_bytes, void *stream) {
     ENTER();
-    CHADQ_REQUIRE(moe_sizes_ok(T, H, F, E, top_k), CHADQ_ERR_SHAPE,
-                  "chadq_moe_ffn_i4g32: T=%d H=%d F=%d E=%d top_k=%d (H, F multiples of 32; E <= 16; top_k <= min(E, 8))", T,
-                  H, F, E, top_k);
-    CHADQ_REQUIRE(x_bf16 && logits && experts && y_bf16, CHADQ_ERR_NULL, "chadq_moe_ffn_i4g32: null pointer");
-    for (int e = 0; e < E; ++e)
-        CHADQ_REQUIRE(experts[e].wg && experts[e].sg && experts[e].wu && experts[e].su && experts[e].wd && experts[e].sd,
-                      CHADQ_ERR_NULL, "chadq_moe_ffn_i4g32: expert %d has a null weight pointer", e);
-    const size_t need = moe_workspace_bytes(T, H, F, E, top_k);
-    CHADQ_REQUIRE(workspace && workspace_bytes >= need, CHADQ_ERR_WORKSPACE,
-                  "chadq_moe_ffn_i4g32: workspace of %zu bytes needed, %zu given", need, workspace ? workspace_bytes : (size_t)0);
-    CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(workspace) && aligned16(y_bf16), CHADQ_ERR_ALIGN,
-                  "chadq_moe_ffn_i4g32: x, y and workspace must be 16-byte aligned");
-    return moe_ffn_i4g32_launch(x_bf16, logits, experts, y_bf16, T, H, F, E, top_k, renorm, workspace, st);
+    return moe_ffn_entry("chadq_moe_ffn_i4g32", false, x_bf16, logits, experts, y_bf16, T, H, F, E, top_k, renorm, workspace,
+                         workspace_bytes, st);
+}
+
+int chadq_moe_ffn_i4g32_tiled(const uint16_t *x_bf16, const float *logits, const chadq_moe_expert_i4g32 *experts,
+                              uint16_t *y_bf16, int T, int H, int F, int E, int top_k, int renorm, void *workspace,
+                              size_t workspace_bytes, void *stream) {
+    ENTER();
+    return moe_ffn_entry("chadq_moe_ffn_i4g32_tiled", true, x_bf16, logits, experts, y_bf16, T, H, F, E, top_k, renorm, workspace,
+                         workspace_bytes, st);
+}
+
+static int repack_entry(const char *name, bool to_tiles, const uint8_t *wp_in, const uint16_t *sc_in, uint8_t *wp_out,
+                        uint16_t *sc_out, int N, int K, hipStream_t st) {
+    CHADQ_REQUIRE(N >= 0 && K >= 0 && N % 32 == 0 && K % 256 == 0, CHADQ_ERR_SHAPE, "%s: N=%d must be a multiple of 32, K=%d of 256",
+                  name, N, K);
+    if (N == 0 || K == 0) return 0;
+    CHADQ_REQUIRE(wp_in && sc_in && wp_out && sc_out, CHADQ_ERR_NULL, "%s: null pointer", name);
+    CHADQ_REQUIRE(wp_in != wp_out && sc_in != sc_out, CHADQ_ERR_SHAPE, "%s: input and output must be different buffers", name);
+    CHADQ_REQUIRE(aligned16(wp_in) && aligned16(sc_in) && aligned16(wp_out) && aligned16(sc_out), CHADQ_ERR_ALIGN,
+                  "%s: all four arrays must be 16-byte aligned", name);
+    return repack_i4g32_tiles_launch(wp_in, sc_in, wp_out, sc_out, N, K, to_tiles, st);
+}
+
+int chadq_repack_i4g32_tiles(const uint8_t *wp, const uint16_t *scale_f16, uint8_t *wp_tiles, uint16_t *scale_tiles, int N, int K,
+                             void *stream) {
+    ENTER();
+    return repack_entry("chadq_repack_i4g32_tiles", true, wp, scale_f16, wp_tiles, scale_tiles, N, K, st);
+}
+
+int chadq_unrepack_i4g32_tiles(const uint8_t *wp_tiles, const uint16_t *scale_tiles, uint8_t *wp, uint16_t *scale_f16, int N, int K,
+                               void *stream) {
+    ENTER();
+    return repack_entry("chadq_unrepack_i4g32_tiles", false, wp_tiles, scale_tiles, wp, scale_f16, N, K, st);
 }
 
 int chadq_embed_i4g32(const int32_t *token, const uint8_t *wp, const uint16_t *scale_f16, float *x, int d, int V, void *stream) {

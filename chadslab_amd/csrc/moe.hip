@@ -40,9 +40,9 @@ int gemm_i4g32_grouped(const GemmGroup *groups, int ngroups, int m_max, int N, i
 bool gemm_skinny_ok(int H, int F);
 int gemm_skinny_tile_rows();
 int gemm_skinny_gateup(const GemmGroup *groups, const int32_t *tiles, const int32_t *tok, int ntiles, int E, int F, int H,
-                       hipStream_t st);
+                       bool tiled, hipStream_t st);
 int gemm_skinny_down(const GemmGroup *groups, const int32_t *tiles, int ntiles, int E, int H, int F, int ksplit, size_t ysplit_stride,
-                     hipStream_t st);
+                     bool tiled, hipStream_t st);
 
 // One workgroup.  Phase 1: softmax + top-k per token.  Phase 2: stable counting sort of the pairs by expert.
 // Phase 3: descriptors.  idx/w may be the caller's arrays (chadq_moe_route) with everything else null.
@@ -287,8 +287,11 @@ int moe_route_launch(const float *logits, int32_t *idx, float *w, int T, int E, 
     return hip_check(hipGetLastError(), "moe_route launch");
 }
 
+// tiled: the experts' weights and scales are in the tile order of chadq_repack_i4g32_tiles (the skinny kernel only)
+bool moe_ffn_tiled_ok(int H, int F) { return gemm_skinny_ok(H, F); }
+
 int moe_ffn_i4g32_launch(const uint16_t *x, const float *logits, const chadq_moe_expert_i4g32 *experts, uint16_t *y,
-                         int T, int H, int F, int E, int top_k, int renorm, void *workspace, hipStream_t st) {
+                         int T, int H, int F, int E, int top_k, int renorm, void *workspace, bool tiled, hipStream_t st) {
     MoeWs ws;
     moe_layout(reinterpret_cast<uint8_t *>(workspace), T, H, F, E, top_k, &ws);
     MoeExperts ex = {};
@@ -309,6 +312,7 @@ int moe_ffn_i4g32_launch(const uint16_t *x, const float *logits, const chadq_moe
         aligned = aligned && aligned16(experts[e].wg) && aligned16(experts[e].sg) && aligned16(experts[e].wu) &&
                   aligned16(experts[e].su) && aligned16(experts[e].wd) && aligned16(experts[e].sd);
     const bool skinny = aligned && gemm_skinny_ok(H, F) && tile_rows <= 128;
+    if (tiled && !skinny) return fail(CHADQ_ERR_ALIGN, "moe_ffn (tiled): weights and scales must be 16-byte aligned, H and F multiples of 256");
     const int route_threads = P <= 256 ? 256 : P <= 512 ? 512 : 1024;
     int rc;
     if (skinny) {  // the router also lists the token tiles; gate/up read the activations through tok
@@ -323,10 +327,10 @@ int moe_ffn_i4g32_launch(const uint16_t *x, const float *logits, const chadq_moe
     }
     if (rc) return rc;
     if (skinny) {
-        rc = gemm_skinny_gateup(ws.groups, ws.tiles, ws.tok, ntiles, E, F, H, st);  // h = bf16(silu(gate) * up), [P,F]
+        rc = gemm_skinny_gateup(ws.groups, ws.tiles, ws.tok, ntiles, E, F, H, tiled, st);  // h = bf16(silu(gate) * up), [P,F]
         if (rc) return rc;
         nsplit = (F % (256 * MOE_KSPLIT) == 0) ? MOE_KSPLIT : 1;
-        rc = gemm_skinny_down(ws.groups, ws.tiles, ntiles, E, H, F, nsplit, (size_t)P * H, st);  // fp32 parts [nsplit][P,H]
+        rc = gemm_skinny_down(ws.groups, ws.tiles, ntiles, E, H, F, nsplit, (size_t)P * H, tiled, st);  // fp32 parts [nsplit][P,H]
         if (rc) return rc;
     } else {
         rc = gemm_i4g32_grouped(ws.groups, 2 * E, m_max, F, H, true, st);  // gate and up: fp32 [P,F] each

@@ -7,6 +7,8 @@ Layouts (this build's choices; the benchmark text fixes only "2 per byte", "grou
                   scale  fp32  [N]
   QWeightInt4G32  packed uint8 [N, K/2]  row-major          byte j of a row = u[2j] | (u[2j+1] << 4), u = q + 8
                   scale  fp16  [N, K/32]                    value = (u - 8) * scale[n, k // 32]
+  QWeightInt4G32Tiles  the same bytes regrouped into contiguous tiles for the mixture-of-experts kernel (a load-time
+                  repack on the device; the row-major form stays the interchange format)
 
 The tensors live wherever the caller puts them; the operators in chadslab_amd.ops want them on the GPU.
 Quantising and packing are load-time tools, not the hot path, and are written with torch tensor ops.
@@ -69,6 +71,28 @@ class QWeightInt4G32:
 
     def to(self, device) -> "QWeightInt4G32":
         return QWeightInt4G32(self.packed.to(device).contiguous(), self.scale.to(device).contiguous())
+
+
+@dataclass
+class QWeightInt4G32Tiles:
+    """An int4 group-32 matrix in tile order (chadq_repack_i4g32_tiles): what ops.moe_ffn streams fastest.  The arrays
+    have the shapes of the row-major container but hold 32-row x 128-k tiles of packed bytes (2 KiB each) and 32-row x
+    8-group blocks of scales (512 B each) contiguously.  Made with ops.to_tiles(); ops.to_rows() is the inverse."""
+    packed: torch.Tensor  # uint8 [N, K/2], tile order
+    scale: torch.Tensor   # float16 [N, K/32], tile order
+
+    def __post_init__(self):
+        QWeightInt4G32(self.packed, self.scale)  # same shape and dtype rules
+        if self.N % 32 or self.K % 256:
+            raise ValueError("tile order needs N % 32 == 0 and K % 256 == 0")
+
+    @property
+    def N(self) -> int:
+        return self.packed.shape[0]
+
+    @property
+    def K(self) -> int:
+        return self.packed.shape[1] * 2
 
 
 def pack_int4(q: torch.Tensor) -> torch.Tensor:

@@ -11,7 +11,7 @@ from typing import Optional, Union
 import torch
 
 from . import _lib
-from .formats import QWeightInt4G32, QWeightInt8
+from .formats import QWeightInt4G32, QWeightInt4G32Tiles, QWeightInt8
 
 QWeight = Union[QWeightInt4G32, QWeightInt8]
 GEMV_MAX_M = 16  # decode batch sizes served by the bandwidth kernel
@@ -152,9 +152,36 @@ def moe_route(logits: torch.Tensor, top_k: int = 2, renorm: bool = True):
 _moe_ws = {}  # (device, stream, bytes) -> workspace tensor, reused between calls on that stream
 
 
+def _repack(w, to_tiles: bool):
+    lib = _lib.load()
+    p, s = _dev(w.packed, "packed", torch.uint8), _dev(w.scale, "scale", torch.float16)
+    if w.N % 32 or w.K % 256:
+        raise ValueError("tile order needs N % 32 == 0 and K % 256 == 0 (N=%d, K=%d)" % (w.N, w.K))
+    po, so = torch.empty_like(p), torch.empty_like(s)
+    fn = lib.chadq_repack_i4g32_tiles if to_tiles else lib.chadq_unrepack_i4g32_tiles
+    _lib.check(fn(p.data_ptr(), s.data_ptr(), po.data_ptr(), so.data_ptr(), w.N, w.K, _stream()),
+               "chadq_repack_i4g32_tiles" if to_tiles else "chadq_unrepack_i4g32_tiles")
+    return po, so
+
+
+def to_tiles(w: QWeightInt4G32) -> QWeightInt4G32Tiles:
+    """Row-major int4 group-32 matrix (on the GPU) -> tile order, for the experts of moe_ffn.  Done once at load time."""
+    if not isinstance(w, QWeightInt4G32):
+        raise TypeError("to_tiles wants a QWeightInt4G32")
+    return QWeightInt4G32Tiles(*_repack(w, True))
+
+
+def to_rows(w: QWeightInt4G32Tiles) -> QWeightInt4G32:
+    """The exact inverse of to_tiles."""
+    if not isinstance(w, QWeightInt4G32Tiles):
+        raise TypeError("to_rows wants a QWeightInt4G32Tiles")
+    return QWeightInt4G32(*_repack(w, False))
+
+
 def moe_ffn(x: torch.Tensor, logits: torch.Tensor, experts, *, top_k: int = 2, renorm: bool = True) -> torch.Tensor:
     """SiLU-gated mixture of experts.  x bf16 [T,H], logits fp32 [T,E]; experts: sequence of (gate, up, down)
-    QWeightInt4G32 triples with gate/up [F,H] and down [H,F].  Returns bf16 [T,H]."""
+    triples with gate/up [F,H] and down [H,F], all QWeightInt4G32 or all QWeightInt4G32Tiles (to_tiles(): the same
+    results bit for bit, faster).  Returns bf16 [T,H]."""
     lib = _lib.load()
     x = _dev(x, "x", torch.bfloat16)
     z = _dev(logits, "logits", torch.float32)
@@ -163,6 +190,10 @@ def moe_ffn(x: torch.Tensor, logits: torch.Tensor, experts, *, top_k: int = 2, r
     if z.shape != (t, e):
         raise ValueError("logits must be [%d,%d]" % (t, e))
     f = experts[0][0].N
+    kinds = {type(m) for tr in experts for m in tr}
+    if kinds not in ({QWeightInt4G32}, {QWeightInt4G32Tiles}):
+        raise TypeError("the experts' matrices must all be QWeightInt4G32 or all QWeightInt4G32Tiles")
+    tiled = kinds == {QWeightInt4G32Tiles}
     arr = (_lib.MoeExpertI4G32 * e)()
     keep = []
     for i, (g, u, d) in enumerate(experts):
@@ -185,6 +216,7 @@ def moe_ffn(x: torch.Tensor, logits: torch.Tensor, experts, *, top_k: int = 2, r
     if ws is None:
         ws = _moe_ws[key] = torch.empty(need, dtype=torch.uint8, device=x.device)
     y = torch.empty(t, h, dtype=torch.bfloat16, device=x.device)
-    _lib.check(lib.chadq_moe_ffn_i4g32(x.data_ptr(), z.data_ptr(), arr, y.data_ptr(), t, h, f, e, top_k, int(renorm),
-                                       ws.data_ptr(), need, _stream()), "chadq_moe_ffn_i4g32")
+    fn = lib.chadq_moe_ffn_i4g32_tiled if tiled else lib.chadq_moe_ffn_i4g32
+    _lib.check(fn(x.data_ptr(), z.data_ptr(), arr, y.data_ptr(), t, h, f, e, top_k, int(renorm), ws.data_ptr(), need, _stream()),
+               "chadq_moe_ffn_i4g32_tiled" if tiled else "chadq_moe_ffn_i4g32")
     return y

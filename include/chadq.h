@@ -161,6 +161,29 @@ int chadq_moe_ffn_i4g32(const uint16_t *x_bf16, const float *logits, const chadq
                         uint16_t *y_bf16, int T, int H, int F, int E, int top_k, int renorm, void *workspace,
                         size_t workspace_bytes, void *stream);
 
+/*
+ * Tile order of int4 group-32 weights: a load-time repack for the experts of chadq_moe_ffn_i4g32_tiled.  The row-major
+ * container (wp [N,K/2], scale [N,K/32]) stays the interchange format; the tiled arrays have the same sizes.
+ *   packed: tile (b = n/32, t = k/128) is 2048 contiguous bytes at ((b*(K/128)) + t) * 2048; inside it row r = n%32
+ *           has its 64 bytes at r*64 as four 16-byte pieces (one scale group each), piece p at position p ^ ((r>>1)&3).
+ *   scales: block (b, c = k/256) is 512 contiguous bytes at ((b*(K/256)) + c) * 512, row r's 8 fp16 at r*16.
+ * N % 32 == 0, K % 256 == 0, all arrays 16-byte aligned, input and output distinct.  unrepack is the exact inverse.
+ * No reference counterpart (the snapshot has no quantized containers): a layout of this build, in FORMAT.md.
+ */
+int chadq_repack_i4g32_tiles(const uint8_t *wp, const uint16_t *scale_f16, uint8_t *wp_tiles, uint16_t *scale_tiles, int N, int K,
+                             void *stream);
+int chadq_unrepack_i4g32_tiles(const uint8_t *wp_tiles, const uint16_t *scale_tiles, uint8_t *wp, uint16_t *scale_f16, int N, int K,
+                               void *stream);
+
+/*
+ * chadq_moe_ffn_i4g32 on experts whose six arrays are in tile order: same arguments, same workspace, same results
+ * bit for bit; the expert weights stream as contiguous 2-KiB tiles instead of 64-byte runs (about 9 % faster at
+ * 256 tokens x 8 experts of 14336 x 4096).  H % 256 == 0 and F % 256 == 0.
+ */
+int chadq_moe_ffn_i4g32_tiled(const uint16_t *x_bf16, const float *logits, const chadq_moe_expert_i4g32 *experts,
+                              uint16_t *y_bf16, int T, int H, int F, int E, int top_k, int renorm, void *workspace,
+                              size_t workspace_bytes, void *stream);
+
 /* ---- decode-step pieces around the GEMVs (benchmark config 4), batch 1 ------------------- */
 /* The position and the current token live in device memory so that one captured HIP graph serves every step.
  * The kernels clamp pos[0] to [0, max_ctx-1] and token[0] to [0, V-1] so that nothing is addressed out of bounds, and

@@ -524,3 +524,73 @@ def test_moe_config3_full_size(ops):
     y = O.bf16_to_f32(bits(ops.moe_ffn(bf16_tensor(xb), torch.from_numpy(logits).to(DEV), dev, top_k=2, renorm=True)))
     ref = O.bf16_to_f32(O.moe_qffn(xb, logits, host, 2, True))
     assert O.rel_l2(y, ref) <= TOL_BF16
+    # the same experts in tile order: the same arithmetic on the same values, so the same bits
+    tiled = [tuple(ops.to_tiles(m) for m in tr) for tr in dev]
+    yt = O.bf16_to_f32(bits(ops.moe_ffn(bf16_tensor(xb), torch.from_numpy(logits).to(DEV), tiled, top_k=2, renorm=True)))
+    assert np.array_equal(yt, y)
+
+
+# ------------------------------------------------------------------ tile order (load-time repack for the experts)
+@pytest.mark.parametrize("n,k", [(32, 256), (64, 512), (96, 1280), (256, 4096), (14336, 4096), (4096, 14336)])
+def test_repack_tiles_bit_exact_and_round_trip(ops, n, k):
+    from chadslab_amd import QWeightInt4G32
+
+    r = rng(5100 + n + k)
+    p = r.integers(0, 256, (n, k // 2), dtype=np.uint8)
+    s = r.integers(0, 65536, (n, k // 32), dtype=np.uint16)  # every bit pattern, NaNs included: the repack moves bytes
+    qw = QWeightInt4G32(torch.from_numpy(p).to(DEV), torch.from_numpy(s).view(torch.float16).to(DEV))
+    tl = ops.to_tiles(qw)
+    wp_t, sc_t = O.tile_int4g32(p, s.view(np.float16))
+    assert np.array_equal(tl.packed.cpu().numpy(), wp_t)
+    assert np.array_equal(tl.scale.view(torch.int16).cpu().numpy().view(np.uint16), sc_t.view(np.uint16))
+    back = ops.to_rows(tl)
+    assert torch.equal(back.packed, qw.packed) and torch.equal(back.scale.view(torch.int16), qw.scale.view(torch.int16))
+
+
+def test_repack_tiles_refuses_bad_shapes_and_aliasing(ops):
+    from chadslab_amd import QWeightInt4G32, _lib
+
+    for n, k in ((48, 256), (32, 128), (32, 288)):
+        qw = QWeightInt4G32(torch.zeros(n, k // 2, dtype=torch.uint8, device=DEV), torch.zeros(n, k // 32, dtype=torch.float16, device=DEV))
+        with pytest.raises(ValueError):
+            ops.to_tiles(qw)
+    lib = _lib.load()
+    a = torch.zeros(32, 128, dtype=torch.uint8, device=DEV)
+    sc = torch.zeros(32, 8, dtype=torch.float16, device=DEV)
+    sc2 = torch.zeros_like(sc)
+    assert lib.chadq_repack_i4g32_tiles(a.data_ptr(), sc.data_ptr(), a.data_ptr(), sc2.data_ptr(), 32, 256, None) == -2  # in place
+    assert lib.chadq_repack_i4g32_tiles(a.data_ptr(), sc.data_ptr(), None, sc2.data_ptr(), 32, 256, None) == -1
+
+
+@pytest.mark.parametrize("t,h,f,e,top_k", [(256, 512, 1024, 8, 2), (64, 256, 256, 1, 1), (130, 256, 512, 16, 4), (300, 256, 768, 2, 2),
+                                           (1200, 256, 256, 4, 4)])
+def test_moe_ffn_tiled_equals_row_major(ops, t, h, f, e, top_k):
+    host, dev = _experts(8800 + t, e, h, f)
+    r = rng(8801 + t)
+    xb = O.f32_to_bf16(r.standard_normal((t, h)).astype(np.float32))
+    logits = r.standard_normal((t, e)).astype(np.float32)
+    y = bits(ops.moe_ffn(bf16_tensor(xb), torch.from_numpy(logits).to(DEV), dev, top_k=top_k, renorm=True))
+    tiled = [tuple(ops.to_tiles(m) for m in tr) for tr in dev]
+    yt = bits(ops.moe_ffn(bf16_tensor(xb), torch.from_numpy(logits).to(DEV), tiled, top_k=top_k, renorm=True))
+    assert np.array_equal(yt, y)
+    ref = O.bf16_to_f32(O.moe_qffn(xb, logits, host, top_k, True))
+    assert O.rel_l2(O.bf16_to_f32(yt), ref) <= TOL_BF16
+
+
+def test_moe_ffn_tiled_refuses_mixed_and_unaligned_shapes(ops):
+    host, dev = _experts(8900, 2, 256, 256)
+    tiled = [tuple(ops.to_tiles(m) for m in tr) for tr in dev]
+    x = torch.zeros(8, 256, dtype=torch.bfloat16, device=DEV)
+    z = torch.zeros(8, 2, device=DEV)
+    with pytest.raises(TypeError):
+        ops.moe_ffn(x, z, [tiled[0], dev[1]], top_k=1)
+    # H = 288 is a multiple of 32 (fine for the row-major entry point) but not of 256: the tiled one refuses it
+    from chadslab_amd import _lib
+    lib = _lib.load()
+    need = lib.chadq_moe_ffn_i4g32_workspace_bytes(8, 288, 256, 1, 1)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=DEV)
+    arr = (_lib.MoeExpertI4G32 * 1)(_lib.MoeExpertI4G32(*[ws.data_ptr()] * 6))
+    y = torch.empty(8, 288, dtype=torch.bfloat16, device=DEV)
+    x2 = torch.zeros(8, 288, dtype=torch.bfloat16, device=DEV)
+    z1 = torch.zeros(8, 1, device=DEV)
+    assert lib.chadq_moe_ffn_i4g32_tiled(x2.data_ptr(), z1.data_ptr(), arr, y.data_ptr(), 8, 288, 256, 1, 1, 1, ws.data_ptr(), need, None) == -2

@@ -442,3 +442,64 @@ def test_sample_topk_draws_the_truncated_softmax():
     assert counts.sum() == draws and set(np.nonzero(counts)[0]) <= set(top.tolist())
     assert np.abs(counts[top] / draws - want).max() <= 1.5 / draws  # a uniform grid of u hits each interval to +-1
 
+
+
+# ------------------------------------------------------------------ tile order (a layout of this build)
+def _tile_loops(wp, sc_u16):
+    """The layout written out address by address: what FORMAT.md and chadq.h say, without numpy reshapes."""
+    n, kh = wp.shape
+    k = kh * 2
+    wt = np.zeros(n * kh, np.uint8)
+    st = np.zeros(n * (k // 32), np.uint16)
+    for row in range(n):
+        b, r = divmod(row, 32)
+        for g in range(k // 32):                      # 16 packed bytes = one scale group
+            t, p = divmod(g, 4)
+            dst = (b * (k // 128) + t) * 2048 + r * 64 + ((p ^ ((r >> 1) & 3)) * 16)
+            wt[dst:dst + 16] = wp[row, g * 16:(g + 1) * 16]
+        for c in range(k // 256):                     # 8 scales = 256 k
+            dst = ((b * (k // 256) + c) * 512 + r * 16) // 2
+            st[dst:dst + 8] = sc_u16[row, c * 8:(c + 1) * 8]
+    return wt.reshape(n, kh), st.reshape(n, k // 32)
+
+
+@pytest.mark.parametrize("n,k", [(32, 256), (64, 512), (96, 768)])
+def test_tile_order_against_address_loops_and_round_trip(n, k):
+    r = np.random.default_rng(600 + n + k)
+    wp = r.integers(0, 256, (n, k // 2), dtype=np.uint8)
+    sc = r.integers(0, 65536, (n, k // 32), dtype=np.uint16)
+    wt, st = O.tile_int4g32(wp, sc.view(np.float16))
+    wl, sl = _tile_loops(wp, sc)
+    assert np.array_equal(wt, wl) and np.array_equal(st.view(np.uint16), sl)
+    a, b = O.untile_int4g32(wt, st)
+    assert np.array_equal(a, wp) and np.array_equal(b.view(np.uint16), sc)
+
+
+def test_tile_order_hand_placed_bytes_and_bijection():
+    n, k = 64, 512
+    # every byte carries its own address, so the tiled array is the permutation itself
+    wp = np.arange(n * k // 2, dtype=np.uint32)
+    tag = (wp % 251).astype(np.uint8).reshape(n, k // 2)
+    wt, _ = O.tile_int4g32(tag, np.zeros((n, k // 32), np.float16))
+    # row 37 (band 1, r = 5, swizzle (5 >> 1) & 3 = 2), scale group 6 (tile 1, piece 2 -> position 0), byte 3 of the group
+    src = 37 * (k // 2) + 6 * 16 + 3
+    dst = (1 * (k // 128) + 1) * 2048 + 5 * 64 + 0 * 16 + 3
+    assert wt.reshape(-1)[dst] == src % 251
+    # row 0, group 0: stays at the very start; row 31 (swizzle 3), group 3 of tile 0 -> position 0 of its 64 bytes
+    assert wt.reshape(-1)[0] == tag[0, 0] and wt.reshape(-1)[31 * 64 + 5] == tag[31, 3 * 16 + 5]
+    idx = np.arange(n * k // 2, dtype=np.int64)
+    lo, hi = (idx & 0xFF).astype(np.uint8).reshape(n, -1), (idx >> 8).astype(np.uint8).reshape(n, -1)
+    perm = O.tile_int4g32(lo, np.zeros((n, k // 32), np.float16))[0].astype(np.int64) + \
+        (O.tile_int4g32(hi, np.zeros((n, k // 32), np.float16))[0].astype(np.int64) << 8)
+    assert np.array_equal(np.sort(perm.reshape(-1)), idx)  # a bijection: every byte appears exactly once
+    s = np.arange(n * k // 32, dtype=np.uint16).reshape(n, k // 32)
+    st = O.tile_int4g32(np.zeros((n, k // 2), np.uint8), s.view(np.float16))[1].view(np.uint16).reshape(-1)
+    assert np.array_equal(np.sort(st), s.reshape(-1))
+    # row 40 (band 1, r = 8), block 1: its eight scales sit at ((1 * 2 + 1) * 512 + 8 * 16) / 2
+    assert np.array_equal(st[(3 * 512 + 128) // 2:(3 * 512 + 128) // 2 + 8], s[40, 8:16])
+
+
+def test_tile_order_refuses_shapes_it_cannot_tile():
+    for n, k in ((48, 256), (32, 128), (32, 288)):
+        with pytest.raises(ValueError):
+            O.tile_int4g32(np.zeros((n, k // 2), np.uint8), np.zeros((n, k // 32), np.float16))
