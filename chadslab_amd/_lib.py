@@ -28,6 +28,8 @@ SIGNATURES = {
     "chadq_gemv_i4g32_splitk_geglu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "chadq_gemv_i4g32_addnorm": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                          c_int, c_void_p]),
+    "chadq_gemv_i4g32_addnorm_geglu": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                         c_int, c_void_p]),
     "chadq_gemv_i8row": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "chadq_gemm_i4g32_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "chadq_gemm_i8row_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),

@@ -64,6 +64,8 @@ int gemv_i4g32_splitk_launch(const uint16_t *, const uint8_t *, const uint16_t *
 int gemv_i4g32_splitk_geglu_launch(const float *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
 int gemv_i4g32_addnorm_launch(const float *, const float *, int, const float *, float, float *, const uint8_t *, const uint16_t *,
                               float *, int, int, hipStream_t);
+int gemv_i4g32_addnorm_geglu_launch(const float *, const float *, int, const float *, float, float *, const uint8_t *, const uint16_t *,
+                                    uint16_t *, int, int, hipStream_t);
 int rope_kv_launch(const float *, const int32_t *, float *, uint16_t *, uint16_t *, int, int, int, float, hipStream_t);
 int attn_mqa_launch(const float *, const uint16_t *, const uint16_t *, const int32_t *, float *, uint16_t *, int, int, int,
                     hipStream_t);
@@ -181,6 +183,24 @@ int chadq_gemv_i4g32_addnorm(const float *res, const float *delta, int n_delta, 
                       aligned16(scale_f16),
                   CHADQ_ERR_ALIGN, "chadq_gemv_i4g32_addnorm: every array must be 16-byte aligned");
     return gemv_i4g32_addnorm_launch(res, delta, delta ? n_delta : 0, norm_w, eps, res_out, wp, scale_f16, y, N, K, st);
+}
+
+int chadq_gemv_i4g32_addnorm_geglu(const float *res, const float *delta, int n_delta, const float *norm_w, float eps,
+                                   float *res_out, const uint8_t *wp, const uint16_t *scale_f16, uint16_t *h_bf16, int N, int K,
+                                   void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(N >= 2 && N % 2 == 0 && K >= 256 && K <= 2048 && K % 256 == 0 && n_delta >= 0 && n_delta <= 4, CHADQ_ERR_SHAPE,
+                  "chadq_gemv_i4g32_addnorm_geglu: N=%d K=%d n_delta=%d (N even, K a multiple of 256 up to 2048, n_delta <= 4)", N, K,
+                  n_delta);
+    CHADQ_REQUIRE((int64_t)N * (K / 2) < ((int64_t)1 << 31), CHADQ_ERR_SHAPE,
+                  "chadq_gemv_i4g32_addnorm_geglu: N*K/2 = %lld bytes exceeds 2^31", (long long)N * (K / 2));
+    CHADQ_REQUIRE(res && norm_w && res_out && wp && scale_f16 && h_bf16 && (delta || n_delta == 0), CHADQ_ERR_NULL,
+                  "chadq_gemv_i4g32_addnorm_geglu: null pointer");
+    CHADQ_REQUIRE(res != res_out, CHADQ_ERR_SHAPE, "chadq_gemv_i4g32_addnorm_geglu: res_out must not be res");
+    CHADQ_REQUIRE(aligned16(res) && aligned16(delta) && aligned16(norm_w) && aligned16(res_out) && aligned16(wp) &&
+                      aligned16(scale_f16),
+                  CHADQ_ERR_ALIGN, "chadq_gemv_i4g32_addnorm_geglu: every array must be 16-byte aligned");
+    return gemv_i4g32_addnorm_geglu_launch(res, delta, delta ? n_delta : 0, norm_w, eps, res_out, wp, scale_f16, h_bf16, N, K, st);
 }
 
 int chadq_gemv_i8row(const float *x, const int8_t *w8, const float *scale, float *y, int M, int N, int K,

@@ -81,7 +81,10 @@ struct GemvPre {
     float eps;
 };
 
-template <int MT, int HP, int S, int RBW, int D, int KC, int XM = 0>
+// YM: what becomes of the sums.  0: y[m,n] fp32.  1 (M = 1): the rows come in pairs (2i, 2i+1) = (gate, up) of feature i
+//     of a gated FFN and the kernel writes h[i] = bf16( gelu_tanh(gate) * up ) through `y` (as uint16_t): the GeGLU of
+//     a decoder layer folded into the projection that produces its inputs.  The tile rows in use (pv) must be even.
+template <int MT, int HP, int S, int RBW, int D, int KC, int XM = 0, int YM = 0>
 __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) void gemv_i4g32_mfma_kernel(
     const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
     float *__restrict__ y, int N, int K, int kspan, int pv, GemvPre pre) {
@@ -339,7 +342,15 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
                     t += reinterpret_cast<const float *>(red)[((wsrc * 64 + lsrc) * MP + p) * 4 + hh * MPASS + m];
                 }
         const int nn = ((blockIdx.x * RBW + un) * (4 / KS) + rb) * pv + rr, mm = p * MPASS + m;
-        if (rr < pv && nn < N && mm < M) y[(size_t)mm * N + nn] = t;
+        if constexpr (YM == 1) {
+            static_assert(YM == 0 || (M == 1 && (C::P % 2) == 0), "gate/up pairs: one activation row, even tiles");
+            // n16 runs fastest over the threads and tiles start at even rows: the up row of a pair sits in the next lane
+            const float up = dpp_f32<0xB1, 0xF>(t);  // quad_perm [1,0,3,2]
+            if (!(rr & 1) && rr + 1 < pv && nn + 1 < N && mm < M)  // mm: the padding rows of a two-row pass write nothing
+                reinterpret_cast<uint16_t *>(y)[nn >> 1] = (uint16_t)f32_to_bf16_bits(gelu_tanh_dev(t) * up);
+        } else {
+            if (rr < pv && nn < N && mm < M) y[(size_t)mm * N + nn] = t;
+        }
     }
 }
 
@@ -766,20 +777,21 @@ static int pick_tile_rows(int N, int P, int tiles_per_wg, int ksplit) {
     return best;
 }
 
-template <int MT, int HP, int S, int RBW, int D, int KC = 4096, int XM = 0>
+template <int MT, int HP, int S, int RBW, int D, int KC = 4096, int XM = 0, int YM = 0>
 static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K,
                        hipStream_t st, int ksplit = 1, GemvPre pre = GemvPre{}) {
     typedef GemvCfg<MT, HP, S, RBW, KC> C;
     static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
     if (!attr_set.load(std::memory_order_acquire)) {
-        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM>),
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM, YM>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::TOTAL));
         attr_set.store(true, std::memory_order_release);
     }
     const int tiles_per_wg = 4 / C::KS * RBW;
-    const int pv = pick_tile_rows(N, C::P, tiles_per_wg, ksplit);
+    int pv = pick_tile_rows(N, C::P, tiles_per_wg, ksplit);
+    if (YM == 1 && (pv & 1)) pv = C::P;  // pairs of rows must not straddle tiles
     const int tiles = (N + pv - 1) / pv;
-    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM>), dim3((tiles + tiles_per_wg - 1) / tiles_per_wg, ksplit),
+    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM, YM>), dim3((tiles + tiles_per_wg - 1) / tiles_per_wg, ksplit),
                        dim3(256 * RBW), C::TOTAL, st, x, wp, sc, y, N, K, K / ksplit, pv, pre);
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma launch");
 }
@@ -894,6 +906,15 @@ int gemv_i4g32_addnorm_launch(const float *res, const float *delta, int n, const
     // many rows: workgroups of 16 waves, so that a compute unit forms the activation vector once, not four times
     if (N >= 8192) return launch_mfma<1, 2, 8, 4, 4, 2048, 2>(nullptr, wp, sc, y, N, K, st, 1, pre);
     return launch_mfma<1, 4, 4, 1, 4, 2048, 2>(nullptr, wp, sc, y, N, K, st, 1, pre);
+}
+
+// The same with the rows of W taken as (gate, up) pairs: h[i] = bf16( gelu_tanh(y[2i]) * y[2i+1] ), N/2 values.
+int gemv_i4g32_addnorm_geglu_launch(const float *res, const float *delta, int n, const float *w, float eps, float *res_out,
+                                    const uint8_t *wp, const uint16_t *sc, uint16_t *h, int N, int K, hipStream_t st) {
+    const GemvPre pre{res, delta, w, res_out, n, eps};
+    float *y = reinterpret_cast<float *>(h);
+    if (N >= 8192) return launch_mfma<1, 2, 8, 4, 4, 2048, 2, 1>(nullptr, wp, sc, y, N, K, st, 1, pre);
+    return launch_mfma<1, 4, 4, 1, 4, 2048, 2, 1>(nullptr, wp, sc, y, N, K, st, 1, pre);
 }
 
 }  // namespace chadq

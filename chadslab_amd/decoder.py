@@ -97,6 +97,14 @@ class QuantDecoder:
         self.ksplit = next((s for s in (4, 2) if c.ffn % (s * 4096) == 0), 1)
         self.gu, self.h, self.dn = z(2 * c.ffn, f32), z(c.ffn, bf16), z(self.ksplit * c.d, f32)
         self.logits = z(c.vocab, f32)
+        # GeGLU folded into the gate+up projection: the kernel wants the gate and the up row of a feature next to each
+        # other, so the decoder keeps a row-interleaved copy of each layer's [2F, d] matrix (made here, once; the
+        # matrices handed in keep the gate-rows-then-up-rows order of the file format)
+        self.fused_geglu = self.fused_norm1
+        if self.fused_geglu:
+            il = torch.arange(2 * c.ffn, device=self.dev).view(2, c.ffn).t().reshape(-1)
+            self.wgu_il = [QWeightInt4G32(L["wgu"].packed.index_select(0, il).contiguous(),
+                                          L["wgu"].scale.index_select(0, il).contiguous()) for L in weights["layers"]]
         # attention with the rotation and the cache write folded in, where its limits allow
         self.fused_attn = c.dh % 16 == 0 and c.max_ctx <= 65536
         if self.fused_attn:
@@ -165,15 +173,21 @@ class QuantDecoder:
                                                      self.pos.data_ptr(), self.part.data_ptr(), self.att.data_ptr(), c.hq, c.dh,
                                                      c.max_ctx, s), "chadq_attn_decode_mqa")
             self._gemv(self.att, L["wo"], self.ao)
-            if self.fused_norm1:  # the second norm folds into the gate+up projection the same way
-                _lib.check(lib.chadq_gemv_i4g32_addnorm(self.x.data_ptr(), self.ao.data_ptr(), 1, L["ln2"].data_ptr(), c.eps,
-                                                        self.x2.data_ptr(), L["wgu"].packed.data_ptr(),
-                                                        L["wgu"].scale.data_ptr(), self.gu.data_ptr(), L["wgu"].N, c.d, s),
-                           "chadq_gemv_i4g32_addnorm")
+            if self.fused_geglu:  # the second norm folds into the gate+up projection, the GeGLU into its epilogue
+                wil = self.wgu_il[li]
+                _lib.check(lib.chadq_gemv_i4g32_addnorm_geglu(self.x.data_ptr(), self.ao.data_ptr(), 1, L["ln2"].data_ptr(), c.eps,
+                                                              self.x2.data_ptr(), wil.packed.data_ptr(), wil.scale.data_ptr(),
+                                                              self.h.data_ptr(), wil.N, c.d, s), "chadq_gemv_i4g32_addnorm_geglu")
                 self.x, self.x2 = self.x2, self.x
-            else:
-                self._norm(self.ao, L["ln2"])
-                self._gemv(self.xn, L["wgu"], self.gu)
+                if self.ksplit > 1:
+                    _lib.check(lib.chadq_gemv_i4g32_splitk(self.h.data_ptr(), L["wd"].packed.data_ptr(), L["wd"].scale.data_ptr(),
+                                                           self.dn.data_ptr(), c.d, c.ffn, self.ksplit, s), "chadq_gemv_i4g32_splitk")
+                else:
+                    self._gemv(self.h, L["wd"], self.dn)
+                pending = self.dn
+                continue
+            self._norm(self.ao, L["ln2"])
+            self._gemv(self.xn, L["wgu"], self.gu)
             if self.ksplit > 1:  # GeGLU folded into the split-K down projection
                 _lib.check(lib.chadq_gemv_i4g32_splitk_geglu(self.gu.data_ptr(), L["wd"].packed.data_ptr(),
                                                              L["wd"].scale.data_ptr(), self.dn.data_ptr(), c.d, c.ffn,

@@ -108,6 +108,16 @@ int chadq_gemv_i4g32_addnorm(const float *res, const float *delta, int n_delta, 
                              const uint8_t *wp, const uint16_t *scale_f16, float *y, int N, int K, void *stream);
 
 /*
+ * chadq_gemv_i4g32_addnorm for the gate/up projection of a GeGLU FFN whose matrix holds the two rows of a feature next
+ * to each other (row 2i = gate of feature i, row 2i+1 = up): instead of the N sums the kernel writes
+ * h[i] = bf16( gelu_tanh(y[2i]) * y[2i+1] ), N/2 values - what chadq_geglu_bf16 would make of them - so that the
+ * down projection reads a bf16 vector and no fp32 gate/up vector is written.  N even; otherwise as above.
+ */
+int chadq_gemv_i4g32_addnorm_geglu(const float *res, const float *delta, int n_delta, const float *norm_w, float eps,
+                                   float *res_out, const uint8_t *wp, const uint16_t *scale_f16, uint16_t *h_bf16, int N, int K,
+                                   void *stream);
+
+/*
  * y[m,n] = scale[n] * sum_k x[m,k] * W[n,k]                                 (config 0)
  * x fp32 [M,K], W int8 [N,K], scale fp32 [N], y fp32 [M,N], 1 <= M <= 16, K % 16 == 0.
  * The weights are streamed once per pair of activation rows (M = 1, 2: once; M = 16: eight times): the fp32

@@ -128,6 +128,44 @@ def test_gemv_addnorm_equals_norm_then_gemv(lib, n, k, nd):
                                          y.data_ptr(), n, k, stream()), "addnorm")
 
 
+@pytest.mark.parametrize("f,k,nd", [(16384, 2048, 1), (16384, 2048, 4), (300, 1024, 0), (4096, 256, 2), (4500, 2048, 1), (1, 256, 1)])
+def test_gemv_addnorm_geglu_equals_addnorm_then_geglu(lib, f, k, nd):
+    # gate+up projection with the GeGLU in its epilogue: rows (2i, 2i+1) = (gate, up) of feature i.  The unfused pair on the
+    # GPU - the same projection on the gate-rows-then-up-rows matrix, then chadq_geglu_bf16 - must give the same bits.
+    r = rng(11 * f + k + nd)
+    u = r.integers(0, 16, (2 * f, k), dtype=np.uint8)
+    packed = (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8)   # rows 0..f-1 gate, f..2f-1 up
+    s = r.lognormal(-5, 0.5, (2 * f, k // 32)).astype(np.float16)
+    il = np.arange(2 * f).reshape(2, f).T.reshape(-1)             # interleaved order: g0, u0, g1, u1, ...
+    res = (r.standard_normal(k) * 2).astype(np.float32)
+    delta = r.standard_normal((max(nd, 1), k)).astype(np.float32)
+    w = (1 + 0.1 * r.standard_normal(k)).astype(np.float32)
+    tp_, ts, tpi, tsi = dev(packed), dev(s), dev(np.ascontiguousarray(packed[il])), dev(np.ascontiguousarray(s[il]))
+    tr, td, tw = dev(res), dev(delta), dev(w)
+    tro, tro2 = torch.zeros(k, dtype=torch.float32, device=DEV), torch.zeros(k, dtype=torch.float32, device=DEV)
+    h = torch.zeros(f, dtype=torch.bfloat16, device=DEV)
+    chk(lib.chadq_gemv_i4g32_addnorm_geglu(tr.data_ptr(), td.data_ptr() if nd else None, nd, tw.data_ptr(), 1e-6, tro.data_ptr(),
+                                           tpi.data_ptr(), tsi.data_ptr(), h.data_ptr(), 2 * f, k, stream()), "addnorm geglu")
+    gu = torch.zeros(2 * f, dtype=torch.float32, device=DEV)
+    h2 = torch.zeros(f, dtype=torch.bfloat16, device=DEV)
+    chk(lib.chadq_gemv_i4g32_addnorm(tr.data_ptr(), td.data_ptr() if nd else None, nd, tw.data_ptr(), 1e-6, tro2.data_ptr(),
+                                     tp_.data_ptr(), ts.data_ptr(), gu.data_ptr(), 2 * f, k, stream()), "addnorm")
+    chk(lib.chadq_geglu_bf16(gu.data_ptr(), h2.data_ptr(), f, stream()), "geglu")
+    assert np.array_equal(tro.cpu().numpy(), tro2.cpu().numpy())
+    assert np.array_equal(bits(h), bits(h2))
+    # and against the CPU restatement
+    want_res = res.copy()
+    for j in range(nd):
+        want_res = want_res + delta[j]
+    xb = O.f32_to_bf16(O.rmsnorm(want_res, w, 1e-6))[None, :]
+    y = O.qgemm_int4g32_f64(xb, packed, s)[0]
+    want = O.gelu_tanh(y[:f]) * y[f:]
+    assert O.rel_l2(O.bf16_to_f32(bits(h)), want) < 6e-3
+    with pytest.raises(ValueError):  # an odd number of rows has no pairs
+        chk(lib.chadq_gemv_i4g32_addnorm_geglu(tr.data_ptr(), None, 0, tw.data_ptr(), 1e-6, tro.data_ptr(), tpi.data_ptr(),
+                                               tsi.data_ptr(), h.data_ptr(), 2 * f - 1, k, stream()), "addnorm geglu")
+
+
 @pytest.mark.parametrize("n,k,ksplit", [(2048, 16384, 4), (100, 8192, 1)])
 def test_gemv_splitk_geglu_equals_geglu_then_gemv(lib, n, k, ksplit):
     r = rng(3 * n + k + ksplit)
