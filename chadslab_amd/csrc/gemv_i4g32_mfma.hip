@@ -355,37 +355,36 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// Eight rows of A per scale group: up to 8 activation rows with one K-part, up to 4 with two.
+// Eight rows of A per scale group: 5 to 8 activation rows in one pass over the unpacked weights.
 //
 // The kernel above gives every lane group j of an MFMA column its own scale group, which leaves four rows of A per
 // group.  Here the two lane-group pairs (0,1) and (2,3) each work on one scale group, eight rows of A per group:
-//   load     as above: lane (n = h*P + r, j) fetches the 16 bytes of group (c*HP + h)*4 + j of weight row r.
-//   exchange v_permlane16_swap on words (0,1) and on words (2,3): lane groups 0 and 1 then hold group 4(c*HP+h)
-//            (pair 0) and the next one (pair 1), lane groups 2 and 3 the two after those - word `half` of each, lane
-//            group j & 1 supplying k 16*half + 8*(j&1) .. +7 of the group.  Two instructions per 16-byte load.
-//   A        row i = 8*g + v (g = which of the pair's two groups, v = h'*MR + m, MR = 8/HP activation rows); real
-//            data where the lane's k-slot group j has j >> 1 == g, zeros elsewhere.
-//   D        lane (n, j) holds rows 8*(j>>1) + 4*(j&1) .. +3 of its column: one scale per lane and pair, four FMAs;
-//            meaningful where the row's K-part h' equals the column's h.
-// Per 16-byte load: 4 MFMAs and 8 scale FMAs.  With HP = 1 that serves 5 to 8 activation rows in one pass (the form
-// above would need 8 and 8): 9.4-9.6 us against 10.4-10.7 at 14336 x 4096 and 8 rows.  HP = 2 would give 3 and 4 rows
-// the load shape of a single row (8 weight rows x 128 contiguous bytes per instruction instead of 16 x 64); it is
-// correct but measured slower than the form above there (8.6 against 8.2 us), so only HP = 1 is dispatched.
-template <int HP, int S, int RBW, int KC>
+//   load     as above with one K-part: lane (r, j) fetches the 16 bytes of group 4c + j of weight row r.
+//   exchange v_permlane16_swap on words (0,1) and on words (2,3): lane groups 0 and 1 then hold group 4c (pair 0) and
+//            group 4c+1 (pair 1), lane groups 2 and 3 hold 4c+2 and 4c+3 - word `half` of each, lane group j & 1
+//            supplying k 16*half + 8*(j&1) .. +7 of the group.  Two instructions per 16-byte load.
+//   A        row i = 8*g + m (g = which of the pair's two groups, m = activation row); real data where the lane's
+//            k-slot group j has j >> 1 == g, zeros elsewhere.
+//   D        lane (r, j) holds activation rows 4*(j&1) .. +3 of weight row r against group 4c + p + 2*(j>>1): one
+//            scale per lane and pair, four FMAs.
+// Per 16-byte load: 4 MFMAs and 8 scale FMAs for up to eight rows (the form above would need 8 and 8): 9.4-9.6 us
+// against 10.4-10.7 at 14336 x 4096 and 8 rows.  (The same regrouping with two K-parts of four rows each - loads of
+// 8 weight rows x 128 contiguous bytes for 3 and 4 activation rows - was built, is correct, and measured slower than
+// the form above there: 8.6 against 8.2 us.)
+template <int S, int RBW, int KC>
 struct GemvPairCfg {
-    static constexpr int P = 16 / HP;
-    static constexpr int MR = 8 / HP;
-    static constexpr int STEPS = KC / (128 * HP);
+    static constexpr int P = 16;
+    static constexpr int MR = 8;
+    static constexpr int STEPS = KC / 128;
     static constexpr int KS = STEPS / S;
     static constexpr int UR = P * 4 / KS;
-    static_assert(HP == 1 || HP == 2, "one or two K-parts");
     static_assert(KS >= 1 && KS <= 4 && KS * S == STEPS, "a chunk of one row block is split over 1, 2 or 4 waves");
     static constexpr int XA_BYTES = STEPS * 2048;  // A operands: [c][pair][half][g][j&1][v] x 16 B
     static constexpr int NX_BYTES = STEPS * 128;   // C operands: [c][pair][j][v%4] fp32
     static constexpr int ZERO_OFF = XA_BYTES + NX_BYTES;
     static constexpr int ZERO_SPAN = 2048;  // lanes off the diagonal add the same per-MFMA offsets (up to 1536) as the others
     static constexpr int SC_OFF = ZERO_OFF + ZERO_SPAN;
-    static constexpr int SC_PPR = S * HP / 2;
+    static constexpr int SC_PPR = S / 2;
     static constexpr int SC_PITCH = SC_PPR * 16 + 16;
     static constexpr int SC_NL = (P * SC_PPR + 63) / 64;
     static constexpr int SC_WAVE = P * SC_PITCH;
@@ -397,20 +396,19 @@ struct GemvPairCfg {
     static_assert((MR * (KC / 8)) % T == 0, "whole rounds of pieces");
 };
 
-template <int MT, int HP, int S, int RBW, int D, int KC>
-__global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((HP == 1 && S == 16) ? 2 : 4))) void gemv_i4g32_mfma_pair_kernel(
+template <int MT, int S, int RBW, int D, int KC>
+__global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(S == 16 ? 2 : 4))) void gemv_i4g32_mfma_pair_kernel(
     const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
     float *__restrict__ y, int N, int K, int pv) {
-    typedef GemvPairCfg<HP, S, RBW, KC> C;
+    typedef GemvPairCfg<S, RBW, KC> C;
     constexpr int M = MT, P = C::P, MR = C::MR, KS = C::KS, T = C::T, XI = C::XI;
-    static_assert(M >= 1 && M <= MR, "eight rows of A per scale group, shared by the K-parts");
-    // HP = 1, S = 16: one 8-wave workgroup per compute unit (its LDS), so a wave may use 256 registers
+    static_assert(M >= 1 && M <= MR, "eight rows of A per scale group");
+    // S = 16: one 8-wave workgroup per compute unit (its LDS), so a wave may use 256 registers
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int unit = wave >> 2, wv = wave & 3;
     const int rbs = wv / KS, ks = wv % KS;
-    const int nl = lane & 15, j = lane >> 4;
-    const int h = nl / P, r = nl % P;
+    const int nl = lane & 15, j = lane >> 4, r = nl;
     const int n0 = ((blockIdx.x * RBW + unit) * (4 / KS) + rbs) * pv;
     const int KH = K >> 1, G = K >> 5;
     const int row = (r < pv && n0 + r < N) ? n0 + r : (n0 < N ? n0 : N - 1);
@@ -419,8 +417,8 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((HP =
 
     for (int o = tid * 16; o < C::ZERO_SPAN; o += T * 16) *reinterpret_cast<u32x4 *>(lds + C::ZERO_OFF + o) = u32x4{0, 0, 0, 0};
 
-    // A operand: lane (i = lane & 15, j) is row 8g + v with g = i >> 3, v = i & 7 = h'*MR + m
-    const bool a_live = ((nl >> 3) == (j >> 1)) && (((nl & 7) % MR) < M);
+    // A operand: lane (i = lane & 15, j) is row 8g + m with g = i >> 3, m = i & 7
+    const bool a_live = ((nl >> 3) == (j >> 1)) && ((nl & 7) < M);
     const uint32_t a_base = a_live ? (uint32_t)(ks * S * 2048 + (j >> 1) * 256 + (j & 1) * 128 + (nl & 7) * 16) : (uint32_t)C::ZERO_OFF;
     const uint32_t a_step = a_live ? 2048u : 0u;
 
@@ -436,14 +434,12 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((HP =
     }
 
     // Piece it = tid + T*q of a chunk: word t = it % 4 of its scale group (the four pieces of a group in one quad of
-    // lanes), activation row m = it / 4 % MR, then K-part hh, pair, g and step from the bits above.  A wave's store
-    // to LDS is four runs of 256 contiguous bytes (conflict free), its load runs of 128 contiguous bytes per row.
-    auto piece = [&](int it, int &t, int &m, int &c, int &hh, int &pr, int &g) {
+    // lanes), activation row m = it / 4 % 8, then pair, g and step from the bits above.  A wave's store to LDS is four
+    // runs of 256 contiguous bytes (conflict free), its load 8 rows x 128 contiguous bytes.
+    auto piece = [&](int it, int &t, int &m, int &c, int &pr, int &g) {
         t = it & 3;
-        m = (it >> 2) % MR;
-        int rest = (it >> 2) / MR;
-        hh = rest % HP;
-        rest /= HP;
+        m = (it >> 2) & 7;
+        const int rest = it >> 5;
         pr = rest & 1;
         g = (rest >> 1) & 1;
         c = rest >> 2;
@@ -454,9 +450,9 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((HP =
         u32x4 xr[XI];
 #pragma unroll
         for (int q = 0; q < XI; ++q) {
-            int t, m, c, hh, pr, g;
-            piece(tid + T * q, t, m, c, hh, pr, g);
-            const int k = kc0 + 32 * ((c * HP + hh) * 4 + g * 2 + pr) + 8 * t;
+            int t, m, c, pr, g;
+            piece(tid + T * q, t, m, c, pr, g);
+            const int k = kc0 + 32 * (c * 4 + g * 2 + pr) + 8 * t;
             xr[q] = u32x4{0, 0, 0, 0};
             if (m < M && k < K) xr[q] = *reinterpret_cast<const u32x4 *>(x + (size_t)m * K + k);
         }
@@ -464,14 +460,14 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((HP =
         u32x4 sv[C::SC_NL];
 #pragma unroll
         for (int l = 0; l < C::SC_NL; ++l) {
-            const int gs = (kc0 >> 5) + ks * S * 4 * HP + spiece[l] * 8;
+            const int gs = (kc0 >> 5) + ks * S * 4 + spiece[l] * 8;
             sv[l] = *reinterpret_cast<const u32x4 *>(sc + ((size_t)srow[l] * G + (gs < G ? gs : 0)));
             if (gs >= G) sv[l] = u32x4{0, 0, 0, 0};
         }
         // 3. the first D weight loads
         u32x4 w[S];
         auto issue_w = [&](int i) {
-            const int gg = (kc0 >> 5) + ((S * ks + i) * HP + h) * 4 + j;
+            const int gg = (kc0 >> 5) + (S * ks + i) * 4 + j;
             w[i] = load_nt_b128(wp + (wrow + (uint32_t)(gg < G ? gg : 0) * 16u));
         };
 #pragma unroll
@@ -485,21 +481,20 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((HP =
             if (srow_l[l] < P) *reinterpret_cast<u32x4 *>(sct + srow_l[l] * C::SC_PITCH + spiece[l] * 16) = sv[l];
 #pragma unroll
         for (int q = 0; q < XI; ++q) {
-            int t, m, c, hh, pr, g;
-            piece(tid + T * q, t, m, c, hh, pr, g);
+            int t, m, c, pr, g;
+            piece(tid + T * q, t, m, c, pr, g);
             uint32_t a[4] = {xr[q].x, xr[q].y, xr[q].z, xr[q].w}, o[4];
             float sum = 0.f;
 #pragma unroll
             for (int e = 0; e < 4; ++e) sum = dot2_bf16(a[e], 0x3F803F80u, sum);
             pair_x8(a, o);
-            const int v = hh * MR + m;
             if (m < M)
-                *reinterpret_cast<u32x4 *>(lds + c * 2048 + (pr * 2 + (t >> 1)) * 512 + g * 256 + (t & 1) * 128 + v * 16) =
+                *reinterpret_cast<u32x4 *>(lds + c * 2048 + (pr * 2 + (t >> 1)) * 512 + g * 256 + (t & 1) * 128 + m * 16) =
                     u32x4{o[0], o[1], o[2], o[3]};
             sum += dpp_f32<0xB1, 0xF>(sum);  // the four pieces of a group sit in four adjacent lanes
             sum += dpp_f32<0x4E, 0xF>(sum);
             if (t == 0 && m < M)
-                *reinterpret_cast<float *>(lds + C::XA_BYTES + ((c * 2 + pr) * 4 + g * 2 + (v >> 2)) * 16 + (v & 3) * 4) =
+                *reinterpret_cast<float *>(lds + C::XA_BYTES + ((c * 2 + pr) * 4 + g * 2 + (m >> 2)) * 16 + (m & 3) * 4) =
                     -kMagicBias * sum;
         }
         __syncthreads();
@@ -524,7 +519,7 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((HP =
 #pragma unroll
             for (int pr = 0; pr < 2; ++pr) {
                 const float s = f16_bits_to_f32(
-                    *reinterpret_cast<const uint16_t *>(sct + r * C::SC_PITCH + ((i * HP + h) * 4 + pr + 2 * (j >> 1)) * 2));
+                    *reinterpret_cast<const uint16_t *>(sct + r * C::SC_PITCH + (i * 4 + pr + 2 * (j >> 1)) * 2));
                 f32x4 d = *reinterpret_cast<const f32x4 *>(lds + C::XA_BYTES + ((2 * c + pr) * 4 + j) * 16);
 #pragma unroll
                 for (int hf = 0; hf < 2; ++hf) {
@@ -540,7 +535,7 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((HP =
         }
     }
 
-    // 6. fold the two scale-group halves, the K-parts and the K-slices
+    // 6. fold the two scale-group halves and the K-slices
     __syncthreads();
     u32x4 *red = reinterpret_cast<u32x4 *>(lds);
     {
@@ -557,13 +552,10 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu((HP =
 #pragma unroll
         for (int k4 = 0; k4 < KS; ++k4)
 #pragma unroll
-            for (int hh = 0; hh < HP; ++hh)
-#pragma unroll
-                for (int g = 0; g < 2; ++g) {
-                    const int v = hh * MR + m;
-                    const int wsrc = un * 4 + rb * KS + k4, lsrc = 16 * (2 * g + (v >> 2)) + hh * P + rr;
-                    t += reinterpret_cast<const float *>(red)[(wsrc * 64 + lsrc) * 4 + (v & 3)];
-                }
+            for (int g = 0; g < 2; ++g) {
+                const int wsrc = un * 4 + rb * KS + k4, lsrc = 16 * (2 * g + (m >> 2)) + rr;
+                t += reinterpret_cast<const float *>(red)[(wsrc * 64 + lsrc) * 4 + (m & 3)];
+            }
         const int nn = ((blockIdx.x * RBW + un) * (4 / KS) + rb) * pv + rr;
         if (rr < pv && nn < N && m < M) y[(size_t)m * N + nn] = t;
     }
@@ -796,19 +788,19 @@ static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc,
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma launch");
 }
 
-template <int MT, int HP, int S, int RBW, int D, int KC = 4096>
+template <int MT, int S, int RBW, int D, int KC = 4096>
 static int launch_pair(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K, hipStream_t st) {
-    typedef GemvPairCfg<HP, S, RBW, KC> C;
+    typedef GemvPairCfg<S, RBW, KC> C;
     static std::atomic<bool> attr_set{false};
     if (!attr_set.load(std::memory_order_acquire)) {
-        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_pair_kernel<MT, HP, S, RBW, D, KC>),
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_pair_kernel<MT, S, RBW, D, KC>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::TOTAL));
         attr_set.store(true, std::memory_order_release);
     }
     const int tiles_per_wg = 4 / C::KS * RBW;
     const int pv = pick_tile_rows(N, C::P, tiles_per_wg, 1);
     const int tiles = (N + pv - 1) / pv;
-    hipLaunchKernelGGL((gemv_i4g32_mfma_pair_kernel<MT, HP, S, RBW, D, KC>), dim3((tiles + tiles_per_wg - 1) / tiles_per_wg), dim3(256 * RBW),
+    hipLaunchKernelGGL((gemv_i4g32_mfma_pair_kernel<MT, S, RBW, D, KC>), dim3((tiles + tiles_per_wg - 1) / tiles_per_wg), dim3(256 * RBW),
                        C::TOTAL, st, x, wp, sc, y, N, K, pv);
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma_pair launch");
 }
@@ -867,16 +859,16 @@ int gemv_i4g32_mfma_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_
                 rc = tall ? launch_mfma<4, 1, 16, 1, 4>(xm, wp, sc, ym, N, K, st) : launch_mfma<4, 1, 8, 1, 8>(xm, wp, sc, ym, N, K, st);
                 break;
             case 5:
-                rc = tall ? launch_pair<5, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_pair<5, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
+                rc = tall ? launch_pair<5, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_pair<5, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
                 break;
             case 6:
-                rc = tall ? launch_pair<6, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_pair<6, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
+                rc = tall ? launch_pair<6, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_pair<6, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
                 break;
             case 7:
-                rc = tall ? launch_pair<7, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_pair<7, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
+                rc = tall ? launch_pair<7, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_pair<7, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
                 break;
             default:
-                rc = tall ? launch_pair<8, 1, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_pair<8, 1, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
+                rc = tall ? launch_pair<8, 16, 2, 4>(xm, wp, sc, ym, N, K, st) : launch_pair<8, 8, 2, 3>(xm, wp, sc, ym, N, K, st);
                 break;
         }
         if (rc != 0) return rc;
