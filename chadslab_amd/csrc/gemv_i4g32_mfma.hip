@@ -226,7 +226,9 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
             ss = wave_sum_to_lane63(ss);
             if (lane == 63) s_ss[wave] = ss;
         }
-        __syncthreads();  // previous chunk's operand reads (or the zero fill) are done
+        // the previous chunk's operand reads are done (first chunk: nothing written below is read before the next
+        // barrier, the zero block included; the norm-folding mode needs the barrier for its sums of squares)
+        if (XN || kc0 != kbeg) __syncthreads();
 #pragma unroll
         for (int l = 0; l < C::SC_NL; ++l)  // wave-private tile
             if (srow_l[l] < P) *reinterpret_cast<u32x4 *>(sct + srow_l[l] * C::SC_PITCH + spiece[l] * 16) = sv[l];
