@@ -143,8 +143,14 @@ static void launch_rows8(const float *x, const int8_t *w8, const float *sc, floa
                        N, K);
 }
 
+bool gemv_i8row_mfma_ok(int M, int K);
+int gemv_i8row_mfma_launch(const float *, const int8_t *, const float *, float *, int, int, int, hipStream_t);
+
 int gemv_i8row_dispatch(const float *x, const int8_t *w8, const float *sc, float *y, int M, int N, int K,
                         hipStream_t st) {
+    // K a multiple of 128: the int8 matrix core, one pass over W for all M (gemv_i8row_mfma.hip); the fp32 kernels
+    // below keep the other row lengths
+    if (N > 0 && gemv_i8row_mfma_ok(M, K)) return gemv_i8row_mfma_launch(x, w8, sc, y, M, N, K, st);
     // <1024-wide chunks per row, rows per wave, activation rows, waves per workgroup>, picked by measurement: eight
     // waves share one copy of the activations; matrices with many rows give a wave 2 or 4 rows
     if (K <= 2048) {

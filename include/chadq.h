@@ -120,9 +120,10 @@ int chadq_gemv_i4g32_addnorm_geglu(const float *res, const float *delta, int n_d
 /*
  * y[m,n] = scale[n] * sum_k x[m,k] * W[n,k]                                 (config 0)
  * x fp32 [M,K], W int8 [N,K], scale fp32 [N], y fp32 [M,N], 1 <= M <= 16, K % 16 == 0.
- * The weights are streamed once per pair of activation rows (M = 1, 2: once; M = 16: eight times): the fp32
- * activations leave registers for two rows' sums only.  Batched decode belongs on the int4 path or on
- * chadq_gemm_i8row_bf16.
+ * K % 128 == 0: the weights are read once for all M rows, on the int8 matrix core; per activation row and 2048 k the
+ * activations are held as three 8-bit fixed-point digits with a power-of-two scale (dropped: < 2^-22 of the block's
+ * largest |x| per element; integer activations below 2^20 stay exact; a non-finite activation makes its row NaN), and
+ * a row's result does not depend on M.  Other K: fp32 arithmetic, the weights streamed once per pair of activation rows.
  */
 int chadq_gemv_i8row(const float *x, const int8_t *w8, const float *scale, float *y, int M, int N, int K,
                      void *stream);

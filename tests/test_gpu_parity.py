@@ -238,15 +238,57 @@ def test_gemv_int8(ops, m, n, k):
     assert O.rel_l2(y, O.qgemv_int8_f64(x, w, s)) <= TOL_F32
 
 
-def test_gemv_int8_integer_exact(ops):
+# K a multiple of 128 runs on the int8 matrix core (activations as three fixed-point digits per 2048 k), one pass over
+# the weights for any M <= 16; other K keep the fp32 kernels
+@pytest.mark.parametrize("m,n,k", [(1, 16384, 2048), (4, 16384, 2048), (5, 16384, 2048), (8, 16384, 2048), (9, 16384, 2048),
+                                   (16, 16384, 2048), (1, 1, 128), (4, 63, 128), (5, 65, 256), (8, 129, 1152), (12, 200, 2176),
+                                   (16, 77, 1920), (3, 4100, 4096), (7, 300, 6144), (16, 130, 8192), (2, 50, 10240),
+                                   (13, 70, 12416)])
+def test_gemv_int8_matrix_core(ops, m, n, k):
+    x, w, s, q8 = i8_case(300 + m + n, m, n, k)
+    y = ops.qgemv(torch.from_numpy(x).to(DEV), q8).cpu().numpy()
+    assert O.rel_l2(y, O.qgemv_int8_f64(x, w, s)) <= TOL_F32
+
+
+@pytest.mark.parametrize("m,n,k", [(2, 300, 2048), (2, 300, 2064), (1, 100, 4096), (5, 333, 4096), (8, 64, 2048), (16, 70, 6144),
+                                   (11, 90, 128)])
+def test_gemv_int8_integer_exact(ops, m, n, k):
     from chadslab_amd import QWeightInt8
 
-    r = rng(21)
-    x = r.integers(-8, 9, (2, 2048)).astype(np.float32)
-    w = r.integers(-127, 128, (300, 2048), dtype=np.int8)
-    q8 = QWeightInt8(torch.from_numpy(w).to(DEV), torch.ones(300, device=DEV))
+    r = rng(21 + m)
+    x = r.integers(-8, 9, (m, k)).astype(np.float32)
+    w = r.integers(-128, 128, (n, k), dtype=np.int8)
+    q8 = QWeightInt8(torch.from_numpy(w).to(DEV), torch.ones(n, device=DEV))
     y = ops.qgemv(torch.from_numpy(x).to(DEV), q8).cpu().numpy()
     assert np.array_equal(y.astype(np.int64), x.astype(np.int64) @ w.astype(np.int64).T)
+
+
+def test_gemv_int8_rows_do_not_depend_on_their_neighbours(ops):
+    """Row m of an M-row call equals the one-row call on x[m] bit for bit (per-row scales, exact integer sums), for
+    every form of the matrix-core kernel (M <= 4, <= 8, <= 16) and across a 2048-k block boundary."""
+    x, w, s, q8 = i8_case(77, 16, 333, 4096)
+    xt = torch.from_numpy(x).to(DEV)
+    one = torch.cat([ops.qgemv(xt[i:i + 1], q8) for i in range(16)]).cpu().numpy()
+    for m in (3, 4, 7, 8, 11, 16):
+        assert np.array_equal(ops.qgemv(xt[:m], q8).cpu().numpy(), one[:m]), m
+
+
+def test_gemv_int8_outliers_zero_rows_and_non_finite_values(ops):
+    x, w, s, q8 = i8_case(78, 6, 200, 4096)
+    x[0, 17] = 3.0e6          # one huge value: the block's fixed-point scale follows it
+    x[1, :] = 0.0             # an all-zero row
+    x[2, 2048:] *= 1.0e-20    # a block of tiny values next to an ordinary one
+    x[3, :] *= 1.0e15
+    y = ops.qgemv(torch.from_numpy(x).to(DEV), q8).cpu().numpy()
+    ref = O.qgemv_int8_f64(x, w, s)
+    for m in range(6):
+        assert O.rel_l2(y[m:m + 1], ref[m:m + 1]) <= TOL_F32 or not ref[m].any(), m
+    assert not y[1].any()
+    x[4, 3000] = np.inf
+    x[5, 5] = np.nan
+    y2 = ops.qgemv(torch.from_numpy(x).to(DEV), q8).cpu().numpy()
+    assert np.isnan(y2[4]).all() and np.isnan(y2[5]).all()   # a non-finite activation makes its own row NaN ...
+    assert np.array_equal(y2[:4], y[:4])                      # ... and no other
 
 
 # ------------------------------------------------------------------ seeded random shapes (ragged edges of every kind)
