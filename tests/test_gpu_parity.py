@@ -322,6 +322,17 @@ def test_random_shapes_int8(ops):
         y1 = ops.qgemv(torch.from_numpy(x[:1]).to(DEV), q8).cpu().numpy()
         ref1 = (x[:1].astype(np.float64) @ (w.astype(np.float64) * s[:, None].astype(np.float64)).T)
         assert O.rel_l2(y1, ref1) <= TOL_F32, ("gemv8", n, k)
+    # the GEMV at every M it takes: K a multiple of 128 (int8 matrix core, all three operand forms, one to six
+    # 2048-blocks) and other K (fp32 kernels), ragged N
+    for case in range(40):
+        m = int(r.integers(1, 17))
+        n = int(r.integers(1, 400)) if case % 4 else int(r.integers(8192, 8400))
+        k = 128 * int(r.integers(1, 90)) if case % 2 else 16 * int(r.integers(1, 300))
+        if n >= 8192:
+            k = min(k, 2048)
+        x, w, s, q8 = i8_case(7000 + case, m, n, k)
+        y = ops.qgemv(torch.from_numpy(x).to(DEV), q8).cpu().numpy()
+        assert y.shape == (m, n) and np.isfinite(y).all() and O.rel_l2(y, O.qgemv_int8_f64(x, w, s)) <= TOL_F32, ("gemv8", m, n, k)
 
 
 # ------------------------------------------------------------------ prefill GEMM (config 2)
