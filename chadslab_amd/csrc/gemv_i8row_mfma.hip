@@ -89,8 +89,8 @@ __global__ __launch_bounds__(512) void gemv_i8row_mfma_kernel(const float *__res
             for (int q = 0; q < 4; ++q) xr[it][q] = *reinterpret_cast<const f32x4 *>(xrow + k + 4 * q);
         }
     };
-    // registers -> fixed point with the block's scale -> three digits -> operand order; returns nothing, leaves the
-    // block's row scales 2^(e-19) (NaN for a non-finite block) in bscale[] of every lane that folds results
+    // registers -> fixed point with the block's scale -> three digits -> operand order; leaves the block's row scales
+    // 2^(e-20) (NaN for a non-finite block) in bscale[] of every lane
     float bscale[C::RES];
     auto stage_x = [&](int sr) {
         float v[C::XIT][16];
