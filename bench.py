@@ -219,6 +219,13 @@ def main():
         b0 = N0 * K0 + N0 * 4 + K0 * 4 + N0 * 4
         extras["gemv_i8row_config0"] = {"us": round(us0, 3), "GBps": round(b0 / us0 * 1e-3, 1),
                                         "frac_hbm_peak": round(b0 / us0 * 1e-3 / HBM_PEAK_GBS, 4)}
+        # labelled extras: the same matrix with 8 and 16 activation rows (one pass over the weights each)
+        for m in (8, 16):
+            xm = torch.from_numpy(r0.standard_normal((m, K0)).astype(np.float32)).to(dev)
+            ym = torch.empty(m, N0, dtype=torch.float32, device=dev)
+            usm = run_steps(lambda i: ops.qgemv(xm, c0[i % N_COPIES], out=ym), *n_side)[0]
+            bm = N0 * K0 + N0 * 4 + m * (K0 * 4 + N0 * 4)
+            extras["gemv_i8row_config0"][f"M{m}_extra"] = {"us": round(usm, 3), "GBps": round(bm / usm * 1e-3, 1)}
         del c0, w0
     if "gemm" in want:
         # config 2: prefill dequant-GEMM, int4 group-32 and int8 per-row
