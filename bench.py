@@ -58,7 +58,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the side measurements")
     ap.add_argument("--extras", default="gemv,int8,gemm,moe,decode",
-                    help="comma list of the side measurements to run (gemv, int8, gemm, moe, decode)")
+                    help="comma list of the side measurements to run (gemv, int8, gemm, moe, decode; moe_ablation adds, "
+                         "to moe, the tile-order call on the two measurement builds of the expert GEMM)")
     ap.add_argument("--short", action="store_true",
                     help="few launches per side measurement: for hardware-counter runs, which serialise every dispatch")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -268,21 +269,22 @@ def main():
                                                    "note": "torch.matmul on bf16 weights, random data: context, not this build's kernel"}
         del wb16, yt
         del x2, y2, q4, q8, p2, s2, x2b, y2b
-    if "moe" in want:
-        # config 3: mixture-of-experts FFN, 8 experts, top-2, 256 tokens (weights random bytes: timing only, parity
-        # is the test suite's job)
+    if "moe" in want or "moe_ablation" in want:
+        # config 3: mixture-of-experts FFN, 8 experts, top-2, 256 tokens, on config 3's own data: PCG64(1003), uniform
+        # nibbles, fp16 group scales ~LogNormal(-5, 0.5), x and the router logits ~N(0,1)
         T3, H3, F3, E3 = 256, 4096, 14336, 8
-        g3 = torch.Generator(device=dev)
-        g3.manual_seed(1003)
+        r3 = np.random.Generator(np.random.PCG64(1003))
 
         def mk(n, k):
-            return QWeightInt4G32(torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev, generator=g3),
-                                  (torch.rand(n, k // 32, device=dev, generator=g3) * 0.01 + 0.002).to(torch.float16))
+            u3 = r3.integers(0, 16, (n, k), dtype=np.uint8)
+            p3 = (u3[:, 0::2] | (u3[:, 1::2] << 4)).astype(np.uint8)
+            s3 = r3.lognormal(-5, 0.5, (n, k // 32)).astype(np.float16)
+            return QWeightInt4G32(torch.from_numpy(p3).to(dev), torch.from_numpy(s3).to(dev))
 
         experts = [(mk(F3, H3), mk(F3, H3), mk(H3, F3)) for _ in range(E3)]
-        x3 = torch.randn(T3, H3, device=dev, generator=g3).to(torch.bfloat16)
-        z3 = torch.randn(T3, E3, device=dev, generator=g3)
-        torch.cuda.synchronize()  # the inputs were generated on the default stream
+        z3 = torch.from_numpy(r3.standard_normal((T3, E3)).astype(np.float32)).to(dev)
+        x3 = torch.from_numpy(r3.standard_normal((T3, H3)).astype(np.float32)).to(torch.bfloat16).to(dev)
+        torch.cuda.synchronize()  # the inputs were copied on the default stream
 
         def time_moe(ex):
             with torch.cuda.stream(stream):
@@ -316,6 +318,24 @@ def main():
         del experts
         torch.cuda.empty_cache()
         extras["moe_ffn_i4g32_config3_tiled"] = moe_entry(time_moe(tiled), "tile order (chadq_repack_i4g32_tiles at load time)")
+        if "moe_ablation" in want:
+            # the same call on the measurement builds (chadslab_amd.build.build_ablations): the expert GEMM with its
+            # arithmetic, or with its weight loads, compiled out - what each half of the loop takes on its own.  The
+            # results of these builds are wrong by construction; only the clock is read.
+            from chadslab_amd.build import ABLATIONS, ablation_path
+
+            main_lib = _lib.load()
+            abl = {"both": extras["moe_ffn_i4g32_config3_tiled"]["us"]}
+            try:
+                for name in ABLATIONS:
+                    if not ablation_path(name).exists():
+                        abl[name] = None
+                        continue
+                    _lib._lib = _lib.open_library(ablation_path(name))
+                    abl[name] = round(time_moe(tiled), 1)
+            finally:
+                _lib._lib = main_lib
+            extras["moe_ffn_i4g32_config3_tiled"]["ablation_us"] = abl
         del tiled, x3, z3
         torch.cuda.empty_cache()
     if "decode" in want:

@@ -72,6 +72,17 @@ class ChadqError(RuntimeError):
     pass
 
 
+def open_library(path) -> ctypes.CDLL:
+    """A build of the library at `path` with the signatures attached (load() for the in-tree one; bench.py also opens
+    the measurement builds of chadslab_amd.build.build_ablations this way)."""
+    lib = ctypes.CDLL(str(path))
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is missing
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
 def load() -> ctypes.CDLL:
     """Loads libchadq.so once and attaches the signatures; raises if it has not been built."""
     global _lib
@@ -81,13 +92,8 @@ def load() -> ctypes.CDLL:
         raise ChadqError(
             "%s not found: build it with `python -m chadslab_amd.build` (there is no fallback path)" % LIB_PATH
         )
-    lib = ctypes.CDLL(str(LIB_PATH))
-    for name, (res, args) in SIGNATURES.items():
-        fn = getattr(lib, name)  # AttributeError if the symbol is missing
-        fn.restype = res
-        fn.argtypes = args
-    _lib = lib
-    return lib
+    _lib = open_library(LIB_PATH)
+    return _lib
 
 
 def check(rc: int, what: str) -> None:

@@ -62,5 +62,33 @@ def build(verbose: bool = True, save_temps: bool = False) -> Path:
     return LIB
 
 
+# Measurement builds of the tile-order expert GEMM (bench.py --extras moe_ablation): the same library with one half of
+# that kernel's loop compiled out, so that each half's share of the time can be measured on its own.  Their results are
+# wrong by construction; nothing but the bench loads them.
+ABLATIONS = {"stream": 1,  # memory traffic without arithmetic
+             "arith": 2}   # arithmetic without weight loads
+
+
+def ablation_path(name: str) -> Path:
+    return PKG / ("libchadq_ablate_%s.so" % name)
+
+
+def build_ablations(verbose: bool = True) -> None:
+    """Needs build() to have run: only gemm_expert_i4g32.hip is recompiled, the other objects are shared."""
+    src = CSRC / "gemm_expert_i4g32.hip"
+    others = [o for o in sorted(OBJ.glob("*.o")) if o.stem != src.stem and not o.stem.startswith("ablate_") and
+              (CSRC / (o.stem + ".hip")).exists()]
+    for name, mode in ABLATIONS.items():
+        obj = OBJ / ("ablate_%s.o" % name)
+        _run([HIPCC, *FLAGS, "-DCHADQ_EXPERT_ABLATE=%d" % mode, "-c", str(src), "-o", str(obj)])
+        tmp = ablation_path(name).with_suffix(".so.tmp")
+        _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, others), str(obj)])
+        os.replace(tmp, ablation_path(name))
+        if verbose:
+            print("built %s" % ablation_path(name))
+
+
 if __name__ == "__main__":
     build(save_temps="--save-temps" in sys.argv)
+    if "--ablations" in sys.argv:
+        build_ablations()

@@ -259,6 +259,9 @@ static int moe_ffn_entry(const char *name, bool tiled, const uint16_t *x_bf16, c
     CHADQ_REQUIRE(moe_sizes_ok(T, H, F, E, top_k), CHADQ_ERR_SHAPE,
                   "%s: T=%d H=%d F=%d E=%d top_k=%d (H, F multiples of 32; E <= 16; top_k <= min(E, 8))", name, T, H, F, E, top_k);
     CHADQ_REQUIRE(!tiled || moe_ffn_tiled_ok(H, F), CHADQ_ERR_SHAPE, "%s: H=%d and F=%d must be multiples of 256", name, H, F);
+    // the tile-order kernel addresses its activation matrices with 32-bit byte offsets
+    CHADQ_REQUIRE(!tiled || (size_t)T * top_k * (size_t)(H > F ? H : F) < ((size_t)1 << 30), CHADQ_ERR_SHAPE,
+                  "%s: T * top_k * max(H, F) = %zu must stay below 2^30", name, (size_t)T * top_k * (size_t)(H > F ? H : F));
     CHADQ_REQUIRE(x_bf16 && logits && experts && y_bf16, CHADQ_ERR_NULL, "%s: null pointer", name);
     for (int e = 0; e < E; ++e)
         CHADQ_REQUIRE(experts[e].wg && experts[e].sg && experts[e].wu && experts[e].su && experts[e].wd && experts[e].sd,

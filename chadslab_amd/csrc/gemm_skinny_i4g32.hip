@@ -46,7 +46,7 @@ constexpr int SK_B_WAVE = SK_NSB * SK_BSLOT;
 constexpr int SK_LDS = SK_A_BYTES + 4 * SK_B_WAVE;
 constexpr int SK_WGS_PER_CU = (2 * SK_LDS <= 160 * 1024) ? 2 : 1;
 
-template <int MODE, int MB, bool TILED>
+template <int MODE, int MB>
 __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, const uint8_t *__restrict__ w0,
                                             const uint16_t *__restrict__ s0, const uint8_t *__restrict__ w1,
                                             const uint16_t *__restrict__ s1, void *__restrict__ yv,
@@ -68,19 +68,14 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
     };
     // weight fetch: DMA instruction i, lane l -> row 16i + l/4, LDS position l%4, which holds 16-byte piece
     // (l%4) ^ ((row >> 1) & 3) of the row's 64 bytes (bank-conflict-free read-back)
-    // TILED: the weights come in tiles (chadq_repack_i4g32_tiles): 32 rows x 128 k of packed bytes are 2 KiB of
-    // contiguous memory already in the order of a slot (row r at r*64, its 16-byte pieces swizzled the same way), and
-    // 32 rows x 8 groups of scales are 512 contiguous bytes.  DMA instruction i is then a linear copy of 1 KiB: the
-    // first or second half of the tile of the wave's row band i/2.
     const uint8_t *wsrc[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int rho = 16 * i + (lane >> 2);
-        if (TILED) wsrc[i] = wptr(32 * (i >> 1)) + (i & 1) * 1024 + lane * 16;  // band start + position inside a tile
-        else wsrc[i] = wptr(rho) + (((lane & 3) ^ ((rho >> 1) & 3)) << 4);
+        wsrc[i] = wptr(rho) + (((lane & 3) ^ ((rho >> 1) & 3)) << 4);
     }
     // scale fetch: lane l -> row l, 8 groups (256 k)
-    const uint16_t *ssrc = TILED ? sptr(lane & 32) + (lane & 31) * 8 : sptr(lane);
+    const uint16_t *ssrc = sptr(lane);
     // read-back: lane (nl, kq), block nb -> row nb*32 + nl; half h of the slot -> piece 2h + kq
     uint32_t brd[2][2];
 #pragma unroll
@@ -129,8 +124,8 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
         const int k = (2 * m < nit) ? kbeg + m * 2 * SK_KI : kbeg;
         uint8_t *bdst = bring + slot * SK_BSLOT;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma16_to_lds(wsrc[i] + (TILED ? (size_t)(k >> 7) * 2048 : (size_t)(k >> 1)), bdst + i * 1024);
-        dma16_to_lds(ssrc + (TILED ? (size_t)(k >> 8) * 256 : (size_t)((k & ~255) >> 5)), bdst + 4096);
+        for (int i = 0; i < 4; ++i) dma16_to_lds(wsrc[i] + (size_t)(k >> 1), bdst + i * 1024);
+        dma16_to_lds(ssrc + (size_t)((k & ~255) >> 5), bdst + 4096);
     };
 
     // one iteration (64 k): weights of half `h` of weight slot `bslot`, activations of stage `stage`
@@ -253,7 +248,7 @@ __device__ __forceinline__ void skinny_body(const uint16_t *__restrict__ x, cons
 // gate/up descriptors' x is the ungathered activation matrix and `pad` the expert's first row in tok, the token of
 // every expert-sorted row.
 // grid: one dimension, decoded in the kernel into n-tile, entry of the tile list and K split (MODE 0 only).
-template <int MODE, bool TILED>
+template <int MODE>
 __global__ __launch_bounds__(256, SK_WGS_PER_CU) void gemm_skinny_i4g32_kernel(const GemmGroup *__restrict__ groups,
                                                                   const int32_t *__restrict__ tiles,
                                                                   const int32_t *__restrict__ tok, int E, int N, int K,
@@ -303,25 +298,25 @@ __global__ __launch_bounds__(256, SK_WGS_PER_CU) void gemm_skinny_i4g32_kernel(c
     }
     const int32_t *rowidx = (MODE == 1 && tok) ? tok + ga.pad : nullptr;
     switch ((rows + 31) >> 5) {
-        case 1: skinny_body<MODE, 1, TILED>(ga.x, w0, s0, w1, s1, y, rowidx, m0, rows, n0, N, K, kbeg, kend, lds); break;
-        case 2: skinny_body<MODE, 2, TILED>(ga.x, w0, s0, w1, s1, y, rowidx, m0, rows, n0, N, K, kbeg, kend, lds); break;
-        default: skinny_body<MODE, 3, TILED>(ga.x, w0, s0, w1, s1, y, rowidx, m0, rows, n0, N, K, kbeg, kend, lds); break;
+        case 1: skinny_body<MODE, 1>(ga.x, w0, s0, w1, s1, y, rowidx, m0, rows, n0, N, K, kbeg, kend, lds); break;
+        case 2: skinny_body<MODE, 2>(ga.x, w0, s0, w1, s1, y, rowidx, m0, rows, n0, N, K, kbeg, kend, lds); break;
+        default: skinny_body<MODE, 3>(ga.x, w0, s0, w1, s1, y, rowidx, m0, rows, n0, N, K, kbeg, kend, lds); break;
     }
 }
 
 bool gemm_skinny_ok(int H, int F) { return H % 256 == 0 && F % 256 == 0; }
 
-template <int MODE, bool TILED>
+template <int MODE>
 static int skinny_launch(const GemmGroup *groups, const int32_t *tiles, const int32_t *tok, int mtiles, int E, int ntiles, int N,
                          int K, int ksplit, size_t ystride, hipStream_t st) {
     static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
     if (!attr_set.load(std::memory_order_acquire)) {
-        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_skinny_i4g32_kernel<MODE, TILED>),
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_skinny_i4g32_kernel<MODE>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS));
         attr_set.store(true, std::memory_order_release);
     }
     const int pairs8 = (mtiles * ksplit + 7) / 8 * 8;  // (list entry, split) pairs, dealt to the 8 XCDs
-    hipLaunchKernelGGL((gemm_skinny_i4g32_kernel<MODE, TILED>), dim3(pairs8 * ntiles), dim3(256), SK_LDS, st, groups, tiles, tok, E, N, K,
+    hipLaunchKernelGGL((gemm_skinny_i4g32_kernel<MODE>), dim3(pairs8 * ntiles), dim3(256), SK_LDS, st, groups, tiles, tok, E, N, K,
                        K / ksplit, ystride, ntiles, mtiles, ksplit);
     return hip_check(hipGetLastError(), "gemm_skinny launch");
 }
@@ -331,16 +326,14 @@ int gemm_skinny_tile_rows() { return SK_MT; }
 // gate/up with the SiLU epilogue: h[P,F] bf16 (through the down descriptors' x pointers).  tok != nullptr: the
 // descriptors address the activations through the token of each row instead of a gathered copy.
 int gemm_skinny_gateup(const GemmGroup *groups, const int32_t *tiles, const int32_t *tok, int ntiles, int E, int F, int H,
-                       bool tiled, hipStream_t st) {
-    return tiled ? skinny_launch<1, true>(groups, tiles, tok, ntiles, E, F / 128, F, H, 1, 0, st)
-                 : skinny_launch<1, false>(groups, tiles, tok, ntiles, E, F / 128, F, H, 1, 0, st);
+                       hipStream_t st) {
+    return skinny_launch<1>(groups, tiles, tok, ntiles, E, F / 128, F, H, 1, 0, st);
 }
 
 // down: fp32 parts [ksplit][P,H]
 int gemm_skinny_down(const GemmGroup *groups, const int32_t *tiles, int ntiles, int E, int H, int F, int ksplit, size_t ysplit_stride,
-                     bool tiled, hipStream_t st) {
-    return tiled ? skinny_launch<0, true>(groups, tiles, nullptr, ntiles, E, H / 256, H, F, ksplit, ysplit_stride, st)
-                 : skinny_launch<0, false>(groups, tiles, nullptr, ntiles, E, H / 256, H, F, ksplit, ysplit_stride, st);
+                     hipStream_t st) {
+    return skinny_launch<0>(groups, tiles, nullptr, ntiles, E, H / 256, H, F, ksplit, ysplit_stride, st);
 }
 
 }  // namespace chadq

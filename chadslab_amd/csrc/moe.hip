@@ -10,6 +10,7 @@
 // dequant-GEMM kernel in grouped mode on a gathered copy of the activations with a separate SiLU kernel; the small
 // kernels here are the router, the gather, the SiLU gate and the weighted combine.
 #include "chadq_common.h"
+#include "expert_prep.h"
 
 namespace chadq {
 
@@ -32,6 +33,12 @@ struct MoeWs {  // workspace carved up on the host
     float *g, *u;        // [P,F]
     uint16_t *h;         // [P,F] bf16
     float *yp;           // [MOE_KSPLIT][P,H] partial down projections
+    // tile-order path: fp16 forms of the two activation matrices (expert_prep.h); xs doubles as the first, one row per token
+    uint16_t *ha;        // [P,F] fp16 form of h
+    float *rsx, *rsh;    // [T] / [P] power of two of each row of xs / ha
+    uint16_t *gxh, *gxl; // [T, H/32 rounded up to 16] group sums of xs, high and low part
+    uint16_t *ghh, *ghl; // [P, F/32 rounded up to 16] group sums of ha
+    uint32_t *rowmax;    // [P] largest finite bf16 magnitude of each row of h
 };
 
 constexpr int MOE_KSPLIT = 4;
@@ -40,16 +47,38 @@ int gemm_i4g32_grouped(const GemmGroup *groups, int ngroups, int m_max, int N, i
 bool gemm_skinny_ok(int H, int F);
 int gemm_skinny_tile_rows();
 int gemm_skinny_gateup(const GemmGroup *groups, const int32_t *tiles, const int32_t *tok, int ntiles, int E, int F, int H,
-                       bool tiled, hipStream_t st);
+                       hipStream_t st);
 int gemm_skinny_down(const GemmGroup *groups, const int32_t *tiles, int ntiles, int E, int H, int F, int ksplit, size_t ysplit_stride,
-                     bool tiled, hipStream_t st);
+                     hipStream_t st);
+// weights in tile order (gemm_expert_i4g32.hip)
+bool gemm_expert_ok(int H, int F);
+int gemm_expert_tile_rows();
+int gemm_expert_down_splits(int F);
+int expert_prep_h_launch(const uint16_t *h, const uint32_t *rowmax, int P, int K, uint16_t *dst, float *rs, uint16_t *ghi, uint16_t *glo,
+                         hipStream_t st);
+int gemm_expert_gateup(const GemmGroup *groups, const int32_t *tiles, const int32_t *tok, int ntiles, int E, int F, int H,
+                       const uint16_t *xa, const float *rs, const uint16_t *ghi, const uint16_t *glo, uint16_t *h, uint32_t *rowmax,
+                       hipStream_t st);
+int gemm_expert_down(const GemmGroup *groups, const int32_t *tiles, int ntiles, int E, int H, int F, const uint16_t *ha,
+                     const float *rs, const uint16_t *ghi, const uint16_t *glo, float *yp, int ksplit, size_t ysplit_stride,
+                     hipStream_t st);
 
-// One workgroup.  Phase 1: softmax + top-k per token.  Phase 2: stable counting sort of the pairs by expert.
+// Workgroup 0.  Phase 1: softmax + top-k per token.  Phase 2: stable counting sort of the pairs by expert.
 // Phase 3: descriptors.  idx/w may be the caller's arrays (chadq_moe_route) with everything else null.
+// Workgroups 1..T (launched for the tile-order path only, prep_x != nullptr): workgroup t+1 turns row t of the
+// activations into the fp16 operands of the tile-order expert GEMM (expert_prep.h) - work that does not depend on the
+// routing and so shares its launch.
 __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict__ logits, int32_t *__restrict__ idx,
                                                          float *__restrict__ w, int T, int E, int top_k, int renorm,
                                                          MoeWs ws, MoeExperts ex, int H, int F,
-                                                         const uint16_t *__restrict__ x_src, int tile_rows, int ntiles_max) {
+                                                         const uint16_t *__restrict__ x_src, int tile_rows, int ntiles_max,
+                                                         const uint16_t *__restrict__ prep_x) {
+    if (blockIdx.x > 0) {
+        __shared__ uint32_t s_pmax[16];
+        const int t = blockIdx.x - 1, g16 = ((H >> 5) + 15) & ~15;
+        prep_row_block(prep_x + (size_t)t * H, H, ws.xs + (size_t)t * H, ws.rsx + t, ws.gxh + (size_t)t * g16, ws.gxl + (size_t)t * g16, s_pmax);
+        return;
+    }
     __shared__ int s_base[MOE_MAX_E];   // rows of expert e seen so far
     __shared__ int s_cnt[16][MOE_MAX_E];  // per-wave counts of every expert in the current chunk
     __shared__ int s_off[MOE_MAX_E + 1];
@@ -118,6 +147,8 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const float *__restrict
             }
     }
     if (!ws.pos) return;  // routing only
+    if (prep_x)
+        for (int p = tid; p < T * top_k; p += B) ws.rowmax[p] = 0u;  // the gate/up kernel takes atomic maxima on these
     __syncthreads();      // idx (global) written by this workgroup is visible to it after the barrier
 
     const int P = T * top_k;
@@ -274,6 +305,15 @@ static size_t moe_layout(uint8_t *base, int T, int H, int F, int E, int top_k, M
     w.u = (float *)take(P * F * 4);
     w.h = (uint16_t *)take(P * F * 2);
     w.yp = (float *)take(P * H * 4 * MOE_KSPLIT);
+    const size_t g16h = (size_t)(((H >> 5) + 15) & ~15), g16f = (size_t)(((F >> 5) + 15) & ~15);
+    w.ha = (uint16_t *)take(P * F * 2);
+    w.rsx = (float *)take(P * 4);
+    w.rsh = (float *)take(P * 4);
+    w.gxh = (uint16_t *)take(P * g16h * 2);
+    w.gxl = (uint16_t *)take(P * g16h * 2);
+    w.ghh = (uint16_t *)take(P * g16f * 2);
+    w.ghl = (uint16_t *)take(P * g16f * 2);
+    w.rowmax = (uint32_t *)take(P * 4);
     if (ws) *ws = w;
     return o;
 }
@@ -283,12 +323,12 @@ size_t moe_workspace_bytes(int T, int H, int F, int E, int top_k) { return moe_l
 int moe_route_launch(const float *logits, int32_t *idx, float *w, int T, int E, int top_k, int renorm, hipStream_t st) {
     MoeWs ws = {};
     MoeExperts ex = {};
-    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 0, st, logits, idx, w, T, E, top_k, renorm, ws, ex, 0, 0, nullptr, 0, 0);
+    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 0, st, logits, idx, w, T, E, top_k, renorm, ws, ex, 0, 0, nullptr, 0, 0, nullptr);
     return hip_check(hipGetLastError(), "moe_route launch");
 }
 
 // tiled: the experts' weights and scales are in the tile order of chadq_repack_i4g32_tiles (the skinny kernel only)
-bool moe_ffn_tiled_ok(int H, int F) { return gemm_skinny_ok(H, F); }
+bool moe_ffn_tiled_ok(int H, int F) { return gemm_expert_ok(H, F); }
 
 int moe_ffn_i4g32_launch(const uint16_t *x, const float *logits, const chadq_moe_expert_i4g32 *experts, uint16_t *y,
                          int T, int H, int F, int E, int top_k, int renorm, void *workspace, bool tiled, hipStream_t st) {
@@ -305,32 +345,42 @@ int moe_ffn_i4g32_launch(const uint16_t *x, const float *logits, const chadq_moe
     }
     const int P = T * top_k;
     const int m_max = P < T ? P : T;  // an expert gets a token at most once
-    const int tile_rows = gemm_skinny_tile_rows(), ntiles = E + P / tile_rows;  // sum over experts of ceil(rows / tile_rows) <= this
+    const int tile_rows = tiled ? gemm_expert_tile_rows() : gemm_skinny_tile_rows();
+    const int ntiles = E + P / tile_rows;  // sum over experts of ceil(rows / tile_rows) <= this
     int nsplit = 1;
-    bool aligned = true;  // the skinny kernel loads scales 16 bytes at a time
+    bool aligned = true;  // the expert kernels load scales 16 bytes at a time
     for (int e = 0; e < E; ++e)
         aligned = aligned && aligned16(experts[e].wg) && aligned16(experts[e].sg) && aligned16(experts[e].wu) &&
                   aligned16(experts[e].su) && aligned16(experts[e].wd) && aligned16(experts[e].sd);
-    const bool skinny = aligned && gemm_skinny_ok(H, F) && tile_rows <= 128;
+    const bool skinny = aligned && (tiled ? gemm_expert_ok(H, F) : gemm_skinny_ok(H, F)) && tile_rows <= 128;
     if (tiled && !skinny) return fail(CHADQ_ERR_ALIGN, "moe_ffn (tiled): weights and scales must be 16-byte aligned, H and F multiples of 256");
     const int route_threads = P <= 256 ? 256 : P <= 512 ? 512 : 1024;
     int rc;
     if (skinny) {  // the router also lists the token tiles; gate/up read the activations through tok
-        hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(route_threads), 0, st, logits, ws.idx, ws.w, T, E, top_k, renorm, ws, ex,
-                           H, F, x, tile_rows, ntiles);
+        hipLaunchKernelGGL(moe_route_kernel, dim3(tiled ? 1 + T : 1), dim3(route_threads), 0, st, logits, ws.idx, ws.w, T, E, top_k, renorm,
+                           ws, ex, H, F, x, tile_rows, ntiles, tiled ? x : nullptr);
         rc = hip_check(hipGetLastError(), "moe route launch");
     } else {
         hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(route_threads), 0, st, logits, ws.idx, ws.w, T, E, top_k, renorm, ws, ex,
-                           H, F, nullptr, 0, 0);
+                           H, F, nullptr, 0, 0, nullptr);
         hipLaunchKernelGGL(moe_gather_kernel, dim3(512), dim3(256), 0, st, x, ws.tok, ws.xs, P, H);
         rc = hip_check(hipGetLastError(), "moe route/gather launch");
     }
     if (rc) return rc;
-    if (skinny) {
-        rc = gemm_skinny_gateup(ws.groups, ws.tiles, ws.tok, ntiles, E, F, H, tiled, st);  // h = bf16(silu(gate) * up), [P,F]
+    if (tiled) {
+        // (the router's launch also made the fp16 form of the activations) gate/up with the SiLU gate, h to fp16, down split over K
+        rc = gemm_expert_gateup(ws.groups, ws.tiles, ws.tok, ntiles, E, F, H, ws.xs, ws.rsx, ws.gxh, ws.gxl, ws.h, ws.rowmax, st);
+        if (rc) return rc;
+        rc = expert_prep_h_launch(ws.h, ws.rowmax, P, F, ws.ha, ws.rsh, ws.ghh, ws.ghl, st);
+        if (rc) return rc;
+        nsplit = gemm_expert_down_splits(F);
+        rc = gemm_expert_down(ws.groups, ws.tiles, ntiles, E, H, F, ws.ha, ws.rsh, ws.ghh, ws.ghl, ws.yp, nsplit, (size_t)P * H, st);
+        if (rc) return rc;
+    } else if (skinny) {
+        rc = gemm_skinny_gateup(ws.groups, ws.tiles, ws.tok, ntiles, E, F, H, st);  // h = bf16(silu(gate) * up), [P,F]
         if (rc) return rc;
         nsplit = (F % (256 * MOE_KSPLIT) == 0) ? MOE_KSPLIT : 1;
-        rc = gemm_skinny_down(ws.groups, ws.tiles, ntiles, E, H, F, nsplit, (size_t)P * H, tiled, st);  // fp32 parts [nsplit][P,H]
+        rc = gemm_skinny_down(ws.groups, ws.tiles, ntiles, E, H, F, nsplit, (size_t)P * H, st);  // fp32 parts [nsplit][P,H]
         if (rc) return rc;
     } else {
         rc = gemm_i4g32_grouped(ws.groups, 2 * E, m_max, F, H, true, st);  // gate and up: fp32 [P,F] each

@@ -76,8 +76,9 @@ class QWeightInt4G32:
 @dataclass
 class QWeightInt4G32Tiles:
     """An int4 group-32 matrix in tile order (chadq_repack_i4g32_tiles): what ops.moe_ffn streams fastest.  The arrays
-    have the shapes of the row-major container but hold 32-row x 128-k tiles of packed bytes (2 KiB each) and 32-row x
-    8-group blocks of scales (512 B each) contiguously.  Made with ops.to_tiles(); ops.to_rows() is the inverse."""
+    have the shapes of the row-major container but hold 32-row x 256-k units of packed bytes (4 KiB each, group-major)
+    and 32-row x 8-group blocks of scales (512 B each) contiguously.  Made with ops.to_tiles(); ops.to_rows() is the
+    inverse.  Scales must stay below 64 in magnitude for the expert kernel."""
     packed: torch.Tensor  # uint8 [N, K/2], tile order
     scale: torch.Tensor   # float16 [N, K/32], tile order
 

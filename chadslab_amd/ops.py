@@ -180,8 +180,8 @@ def to_rows(w: QWeightInt4G32Tiles) -> QWeightInt4G32:
 
 def moe_ffn(x: torch.Tensor, logits: torch.Tensor, experts, *, top_k: int = 2, renorm: bool = True) -> torch.Tensor:
     """SiLU-gated mixture of experts.  x bf16 [T,H], logits fp32 [T,E]; experts: sequence of (gate, up, down)
-    triples with gate/up [F,H] and down [H,F], all QWeightInt4G32 or all QWeightInt4G32Tiles (to_tiles(): the same
-    results bit for bit, faster).  Returns bf16 [T,H]."""
+    triples with gate/up [F,H] and down [H,F], all QWeightInt4G32 or all QWeightInt4G32Tiles (to_tiles(): faster, fp16
+    instead of bf16 dequantised weights, so the same results within rounding).  Returns bf16 [T,H]."""
     lib = _lib.load()
     x = _dev(x, "x", torch.bfloat16)
     z = _dev(logits, "logits", torch.float32)

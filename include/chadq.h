@@ -175,9 +175,10 @@ int chadq_moe_ffn_i4g32(const uint16_t *x_bf16, const float *logits, const chadq
 /*
  * Tile order of int4 group-32 weights: a load-time repack for the experts of chadq_moe_ffn_i4g32_tiled.  The row-major
  * container (wp [N,K/2], scale [N,K/32]) stays the interchange format; the tiled arrays have the same sizes.
- *   packed: tile (b = n/32, t = k/128) is 2048 contiguous bytes at ((b*(K/128)) + t) * 2048; inside it row r = n%32
- *           has its 64 bytes at r*64 as four 16-byte pieces (one scale group each), piece p at position p ^ ((r>>1)&3).
- *   scales: block (b, c = k/256) is 512 contiguous bytes at ((b*(K/256)) + c) * 512, row r's 8 fp16 at r*16.
+ *   packed: unit (b = n/32, c = k/256) is 4096 contiguous bytes at ((b*(K/256)) + c) * 4096; inside it the 16-byte
+ *           piece (one scale group) of row r = n%32 and group g = (k%256)/32 sits at (g*32 + r) * 16.
+ *   scales: block (b, c) is 512 contiguous bytes at ((b*(K/256)) + c) * 512; the scale of row r and group g sits at
+ *           ((g%2)*32 + r) * 8 + (g/2) * 2.
  * N % 32 == 0, K % 256 == 0, all arrays 16-byte aligned, input and output distinct.  unrepack is the exact inverse.
  * No reference counterpart (the snapshot has no quantized containers): a layout of this build, in FORMAT.md.
  */
@@ -187,9 +188,15 @@ int chadq_unrepack_i4g32_tiles(const uint8_t *wp_tiles, const uint16_t *scale_ti
                                void *stream);
 
 /*
- * chadq_moe_ffn_i4g32 on experts whose six arrays are in tile order: same arguments, same workspace, same results
- * bit for bit; the expert weights stream as contiguous 2-KiB tiles instead of 64-byte runs (9 to 20 % faster at
- * 256 tokens x 8 experts of 14336 x 4096).  H % 256 == 0 and F % 256 == 0.
+ * chadq_moe_ffn_i4g32 on experts whose six arrays are in tile order: same arguments, same workspace.  Each load of the
+ * expert kernel then reads 1 KiB of consecutive memory straight into registers, and the arithmetic is fp16 instead of
+ * bf16: activations (and the gated intermediate h, after its bf16 rounding) are scaled per row by a power of two into
+ * fp16's range - exact for bf16 inputs of any magnitude, the factor is undone on the fp32 result - and a weight enters
+ * the matrix core as fp16(u * scale), the zero point as a separate exact term per scale group.  The results agree with
+ * chadq_moe_ffn_i4g32 within rounding (they are the closer of the two to a float64 evaluation: fp16 keeps 3 more bits
+ * of the dequantised weight than bf16), not bit for bit.  About 20 % faster at 256 tokens x 8 experts of 14336 x 4096.
+ * H % 256 == 0 and F % 256 == 0; scales must be below 64 in magnitude (1024 * scale has to be a finite fp16);
+ * T * top_k * max(H, F) < 2^30.
  */
 int chadq_moe_ffn_i4g32_tiled(const uint16_t *x_bf16, const float *logits, const chadq_moe_expert_i4g32 *experts,
                               uint16_t *y_bf16, int T, int H, int F, int E, int top_k, int renorm, void *workspace,

@@ -89,11 +89,11 @@ def unpack_int4(wp: np.ndarray) -> np.ndarray:
 def tile_int4g32(wp: np.ndarray, scale_f16: np.ndarray):
     """Row-major (wp uint8 [N,K/2], scale fp16 [N,K/32]) -> tile order, same shapes.
 
-    BUILD CHOICE (a layout of this build, no reference counterpart).  Packed bytes: the matrix is cut into tiles of
-    32 rows x 128 k (64 bytes per row); tile (b, t) occupies 2048 contiguous bytes at ((b * K/128) + t) * 2048, row r
-    at r * 64 inside it, and the row's four 16-byte pieces (one scale group each) are stored with piece p at position
-    p ^ ((r >> 1) & 3).  Scales: blocks of 32 rows x 8 groups, block (b, c) at ((b * K/256) + c) * 512 bytes, row r's
-    eight scales at r * 16.  N % 32 == 0, K % 256 == 0.
+    BUILD CHOICE (a layout of this build, no reference counterpart).  Packed bytes: the matrix is cut into units of
+    32 rows x 256 k; unit (b, c) occupies 4096 contiguous bytes at ((b * K/256) + c) * 4096, and inside it the 16-byte
+    piece (one scale group) of row r and group g sits at (g * 32 + r) * 16.  Scales: block (b, c) = the same 32 rows x
+    8 groups is 512 bytes at ((b * K/256) + c) * 512, the scale of row r and group g at
+    ((g % 2) * 32 + r) * 8 + (g // 2) * 2.  N % 32 == 0, K % 256 == 0.
     """
     wp = np.ascontiguousarray(wp, dtype=np.uint8)
     sc = np.ascontiguousarray(scale_f16).view(np.uint16)
@@ -101,10 +101,8 @@ def tile_int4g32(wp: np.ndarray, scale_f16: np.ndarray):
     k = kh * 2
     if n % 32 or k % 256 or sc.shape != (n, k // GROUP):
         raise ValueError("tile order needs N % 32 == 0, K % 256 == 0 and scales [N,K/32]")
-    x = wp.reshape(n // 32, 32, k // 128, 4, 16).transpose(0, 2, 1, 3, 4)  # [band, tile, row, piece, 16 B]
-    swz = (np.arange(32)[:, None] >> 1 & 3) ^ np.arange(4)[None, :]         # position q of row r holds piece q ^ m(r)
-    tiles = np.take_along_axis(x, swz[None, None, :, :, None], axis=3)
-    st = sc.reshape(n // 32, 32, k // 256, 8).transpose(0, 2, 1, 3)          # [band, block, row, 8]
+    tiles = wp.reshape(n // 32, 32, k // 256, 8, 16).transpose(0, 2, 3, 1, 4)   # [band, unit, group, row, 16 B]
+    st = sc.reshape(n // 32, 32, k // 256, 4, 2).transpose(0, 2, 4, 1, 3)       # [band, unit, parity, row, group // 2]
     return (np.ascontiguousarray(tiles).reshape(n, kh),
             np.ascontiguousarray(st).reshape(n, k // GROUP).view(np.float16))
 
@@ -117,10 +115,8 @@ def untile_int4g32(wp_tiles: np.ndarray, scale_tiles: np.ndarray):
     k = kh * 2
     if n % 32 or k % 256 or stl.shape != (n, k // GROUP):
         raise ValueError("tile order needs N % 32 == 0, K % 256 == 0 and scales [N,K/32]")
-    x = wt.reshape(n // 32, k // 128, 32, 4, 16)
-    swz = (np.arange(32)[:, None] >> 1 & 3) ^ np.arange(4)[None, :]         # the swizzle is its own inverse
-    rows = np.take_along_axis(x, swz[None, None, :, :, None], axis=3).transpose(0, 2, 1, 3, 4)
-    sr = stl.reshape(n // 32, k // 256, 32, 8).transpose(0, 2, 1, 3)
+    rows = wt.reshape(n // 32, k // 256, 8, 32, 16).transpose(0, 3, 1, 2, 4)    # [band, row, unit, group, 16 B]
+    sr = stl.reshape(n // 32, k // 256, 2, 32, 4).transpose(0, 3, 1, 4, 2)      # [band, row, unit, group // 2, parity]
     return (np.ascontiguousarray(rows).reshape(n, kh),
             np.ascontiguousarray(sr).reshape(n, k // GROUP).view(np.float16))
 

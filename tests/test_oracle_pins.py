@@ -446,7 +446,8 @@ def test_sample_topk_draws_the_truncated_softmax():
 
 # ------------------------------------------------------------------ tile order (a layout of this build)
 def _tile_loops(wp, sc_u16):
-    """The layout written out address by address: what FORMAT.md and chadq.h say, without numpy reshapes."""
+    """The layout written out address by address, without numpy reshapes: unit (band, 256 k) of 4096 bytes, a group's
+    32 rows next to each other; scale block of 512 bytes, per row the even groups' scales, 256 bytes on the odd ones'."""
     n, kh = wp.shape
     k = kh * 2
     wt = np.zeros(n * kh, np.uint8)
@@ -454,12 +455,11 @@ def _tile_loops(wp, sc_u16):
     for row in range(n):
         b, r = divmod(row, 32)
         for g in range(k // 32):                      # 16 packed bytes = one scale group
-            t, p = divmod(g, 4)
-            dst = (b * (k // 128) + t) * 2048 + r * 64 + ((p ^ ((r >> 1) & 3)) * 16)
+            c, g8 = divmod(g, 8)
+            dst = (b * (k // 256) + c) * 4096 + (g8 * 32 + r) * 16
             wt[dst:dst + 16] = wp[row, g * 16:(g + 1) * 16]
-        for c in range(k // 256):                     # 8 scales = 256 k
-            dst = ((b * (k // 256) + c) * 512 + r * 16) // 2
-            st[dst:dst + 8] = sc_u16[row, c * 8:(c + 1) * 8]
+            dsts = ((b * (k // 256) + c) * 512 + ((g8 % 2) * 32 + r) * 8 + (g8 // 2) * 2) // 2
+            st[dsts] = sc_u16[row, g]
     return wt.reshape(n, kh), st.reshape(n, k // 32)
 
 
@@ -481,12 +481,12 @@ def test_tile_order_hand_placed_bytes_and_bijection():
     wp = np.arange(n * k // 2, dtype=np.uint32)
     tag = (wp % 251).astype(np.uint8).reshape(n, k // 2)
     wt, _ = O.tile_int4g32(tag, np.zeros((n, k // 32), np.float16))
-    # row 37 (band 1, r = 5, swizzle (5 >> 1) & 3 = 2), scale group 6 (tile 1, piece 2 -> position 0), byte 3 of the group
-    src = 37 * (k // 2) + 6 * 16 + 3
-    dst = (1 * (k // 128) + 1) * 2048 + 5 * 64 + 0 * 16 + 3
+    # row 37 (band 1, r = 5), scale group 14 (unit 1, group 6 of it), byte 3 of the group
+    src = 37 * (k // 2) + 14 * 16 + 3
+    dst = (1 * (k // 256) + 1) * 4096 + (6 * 32 + 5) * 16 + 3
     assert wt.reshape(-1)[dst] == src % 251
-    # row 0, group 0: stays at the very start; row 31 (swizzle 3), group 3 of tile 0 -> position 0 of its 64 bytes
-    assert wt.reshape(-1)[0] == tag[0, 0] and wt.reshape(-1)[31 * 64 + 5] == tag[31, 3 * 16 + 5]
+    # row 0, group 0 stays at the very start; row 31, group 0 ends the first 512 bytes; row 0, group 1 follows it
+    assert wt.reshape(-1)[0] == tag[0, 0] and wt.reshape(-1)[31 * 16 + 5] == tag[31, 5] and wt.reshape(-1)[512 + 2] == tag[0, 16 + 2]
     idx = np.arange(n * k // 2, dtype=np.int64)
     lo, hi = (idx & 0xFF).astype(np.uint8).reshape(n, -1), (idx >> 8).astype(np.uint8).reshape(n, -1)
     perm = O.tile_int4g32(lo, np.zeros((n, k // 32), np.float16))[0].astype(np.int64) + \
@@ -495,8 +495,9 @@ def test_tile_order_hand_placed_bytes_and_bijection():
     s = np.arange(n * k // 32, dtype=np.uint16).reshape(n, k // 32)
     st = O.tile_int4g32(np.zeros((n, k // 2), np.uint8), s.view(np.float16))[1].view(np.uint16).reshape(-1)
     assert np.array_equal(np.sort(st), s.reshape(-1))
-    # row 40 (band 1, r = 8), block 1: its eight scales sit at ((1 * 2 + 1) * 512 + 8 * 16) / 2
-    assert np.array_equal(st[(3 * 512 + 128) // 2:(3 * 512 + 128) // 2 + 8], s[40, 8:16])
+    # row 40 (band 1, r = 8), unit 1: its even groups' scales at (3 * 512 + 8 * 8) / 2, the odd ones' 128 entries on
+    at = (3 * 512 + 8 * 8) // 2
+    assert np.array_equal(st[at:at + 4], s[40, 8:16:2]) and np.array_equal(st[at + 128:at + 132], s[40, 9:16:2])
 
 
 def test_tile_order_refuses_shapes_it_cannot_tile():
