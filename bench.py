@@ -155,6 +155,7 @@ def main():
     n_dec = 4 if args.short else 64
     results = {}
     parity = {}
+    host = {}  # host copies of the side measurements' inputs, for the CPU legs
     for m in (1, 4, 8):
         if m != 1 and "gemv" not in want:
             continue
@@ -205,15 +206,25 @@ def main():
                 "us": round(us_rd, 3), "GBps": round(nread / us_rd * 1e-3, 1), "bytes": int(nread),
                 "note": "loads only (bench_probe.hip), rotating buffers: the machine's ceiling for a read of this size"}
             del flat, pout
+            # a dependent launch of a kernel that does nothing, replayed from a graph like everything else here
+            plib.bench_probe_empty.restype = ctypes.c_int
+            plib.bench_probe_empty.argtypes = [ctypes.c_void_p]
+
+            def empty(i):
+                if plib.bench_probe_empty(torch.cuda.current_stream().cuda_stream):
+                    raise RuntimeError("bench_probe_empty failed")
+
+            extras["launch_floor_us"] = {"us": round(run_steps(empty, *n_side)[0], 3),
+                                         "note": "an empty kernel (bench_probe.hip) per step, dependent launches in a replayed graph"}
     del copies
 
     if "int8" in want:
         # config 0: int8 per-row GEMV
         N0, K0 = 16384, 2048
         r0 = np.random.Generator(np.random.PCG64(1000))
-        x0 = torch.from_numpy(r0.standard_normal((1, K0)).astype(np.float32)).to(dev)
-        w0 = torch.from_numpy(r0.integers(-127, 128, (N0, K0), dtype=np.int8)).to(dev)
-        s0 = torch.from_numpy(r0.uniform(0.001, 0.02, N0).astype(np.float32)).to(dev)
+        host["cfg0"] = (r0.standard_normal((1, K0)).astype(np.float32), r0.integers(-127, 128, (N0, K0), dtype=np.int8),
+                        r0.uniform(0.001, 0.02, N0).astype(np.float32))
+        x0, w0, s0 = (torch.from_numpy(a).to(dev) for a in host["cfg0"])
         c0 = [QWeightInt8(w0.clone(), s0.clone()) for _ in range(N_COPIES)]
         y0 = torch.empty(1, N0, dtype=torch.float32, device=dev)
         us0 = run_steps(lambda i: ops.qgemv(x0, c0[i % N_COPIES], out=y0), *n_side)[0]
@@ -232,13 +243,15 @@ def main():
         # config 2: prefill dequant-GEMM, int4 group-32 and int8 per-row
         M2, N2, K2 = 512, 4096, 4096
         r2 = np.random.Generator(np.random.PCG64(1002))
-        p2 = torch.from_numpy(r2.integers(0, 256, (N2, K2 // 2), dtype=np.uint8)).to(dev)
-        s2 = torch.from_numpy(r2.lognormal(-5, 0.5, (N2, K2 // 32)).astype(np.float16)).to(dev)
-        x2 = torch.from_numpy(r2.standard_normal((M2, K2)).astype(np.float32)).to(torch.bfloat16).to(dev)
+        p2h, s2h = r2.integers(0, 256, (N2, K2 // 2), dtype=np.uint8), r2.lognormal(-5, 0.5, (N2, K2 // 32)).astype(np.float16)
+        x2h = r2.standard_normal((M2, K2)).astype(np.float32)
+        w8h, s8h = r2.integers(-127, 128, (N2, K2), dtype=np.int8), r2.uniform(0.001, 0.02, N2).astype(np.float32)
+        host["cfg2"] = (x2h, p2h, s2h, w8h, s8h)
+        p2, s2 = torch.from_numpy(p2h).to(dev), torch.from_numpy(s2h).to(dev)
+        x2 = torch.from_numpy(x2h).to(torch.bfloat16).to(dev)
         y2 = torch.empty(M2, N2, dtype=torch.bfloat16, device=dev)
         q4 = QWeightInt4G32(p2, s2)
-        q8 = QWeightInt8(torch.from_numpy(r2.integers(-127, 128, (N2, K2), dtype=np.int8)).to(dev),
-                         torch.from_numpy(r2.uniform(0.001, 0.02, N2).astype(np.float32)).to(dev))
+        q8 = QWeightInt8(torch.from_numpy(w8h).to(dev), torch.from_numpy(s8h).to(dev))
         flop = 2.0 * M2 * N2 * K2
         for name, qw in (("gemm_i4g32_config2", q4), ("gemm_i8row_config2", q8)):
             usg = run_steps(lambda i: ops.qgemm(x2, qw, out=y2), *n_gemm)[0]
@@ -275,15 +288,21 @@ def main():
         T3, H3, F3, E3 = 256, 4096, 14336, 8
         r3 = np.random.Generator(np.random.PCG64(1003))
 
+        first3 = []  # expert 0's host arrays, for the CPU leg
+
         def mk(n, k):
             u3 = r3.integers(0, 16, (n, k), dtype=np.uint8)
             p3 = (u3[:, 0::2] | (u3[:, 1::2] << 4)).astype(np.uint8)
             s3 = r3.lognormal(-5, 0.5, (n, k // 32)).astype(np.float16)
+            if len(first3) < 6:
+                first3.extend([p3, s3])
             return QWeightInt4G32(torch.from_numpy(p3).to(dev), torch.from_numpy(s3).to(dev))
 
         experts = [(mk(F3, H3), mk(F3, H3), mk(H3, F3)) for _ in range(E3)]
-        z3 = torch.from_numpy(r3.standard_normal((T3, E3)).astype(np.float32)).to(dev)
-        x3 = torch.from_numpy(r3.standard_normal((T3, H3)).astype(np.float32)).to(torch.bfloat16).to(dev)
+        z3h, x3h = r3.standard_normal((T3, E3)).astype(np.float32), r3.standard_normal((T3, H3)).astype(np.float32)
+        host["cfg3"] = (x3h, z3h, tuple(first3))
+        z3 = torch.from_numpy(z3h).to(dev)
+        x3 = torch.from_numpy(x3h).to(torch.bfloat16).to(dev)
         torch.cuda.synchronize()  # the inputs were copied on the default stream
 
         def time_moe(ex):
@@ -391,10 +410,22 @@ def main():
             b4.record(stream)
             torch.cuda.synchronize()
         extras["decode_step_config4"]["us_per_token_sampling_top50"] = round(a4.elapsed_time(b4) * 1000.0 / n_dec, 1)
+        if not args.no_cpu:  # two layers and the table go back to the host for the CPU leg
+
+            def to_host(q):
+                return q.packed.cpu().numpy(), q.scale.cpu().numpy()
+
+            host["cfg4"] = {"layers": [{k: (to_host(v) if hasattr(v, "packed") else v.cpu().numpy()) for k, v in L.items()}
+                                       for L in w4["layers"][:2]],
+                            "lnf": w4["lnf"].cpu().numpy(), "emb": to_host(w4["emb"]), "cfg": cfg4}
         del dec, w4
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ CPU baseline (rank 0, N=1)
+    # The reference snapshot holds no implementation of this path, so what is timed is this build's numpy oracle, written
+    # the way a plain numpy runtime would be: (i) dequantise to fp32, then matmul - what a naive runtime pays per call -
+    # and (ii) the matmul alone on weights dequantised beforehand - its best case.  Headline config in cpu_baseline,
+    # the other configs under cpu_baseline.configs, each on a bounded sample.
     cpu = None
     if not args.no_cpu:
         from oracle import chadq_oracle as O
@@ -405,30 +436,109 @@ def main():
             threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
         except Exception:
             threads = os.cpu_count() or 1
+
+        def med(fn, reps, warm=1):
+            for _ in range(warm):
+                fn()
+            ts = []
+            for _ in range(reps):
+                t0 = time.perf_counter()
+                fn()
+                ts.append(time.perf_counter() - t0)
+            return float(np.median(ts))
+
         xb = O.f32_to_bf16(x_np[1])
         t0 = time.perf_counter()
         O.qgemv_int4g32(xb, packed, scale)
         first = time.perf_counter() - t0
-        reps = int(min(40, max(3, 15.0 / max(first, 1e-3))))
-        times = []
-        for _ in range(reps):
-            t0 = time.perf_counter()
-            O.qgemv_int4g32(xb, packed, scale)
-            times.append(time.perf_counter() - t0)
-        med = float(np.median(times))
+        reps = int(min(40, max(3, 8.0 / max(first, 1e-3))))
+        t_dq = med(lambda: O.qgemv_int4g32(xb, packed, scale), reps, 0)
         wd = O.dequant_int4g32(packed, scale)
         xf = O.bf16_to_f32(xb)
-        t2 = []
-        for _ in range(10):
-            t0 = time.perf_counter()
-            xf @ wd.T
-            t2.append(time.perf_counter() - t0)
+        t_pre = med(lambda: xf @ wd.T, 10)
+        del wd
+        per_cfg = {}
+        if "cfg0" in host:
+            x0h, w0h, s0h = host["cfg0"]
+            b0h = w0h.size + 2 * s0h.size * 4 + x0h.size * 4
+            t_a = med(lambda: O.qgemv_int8(x0h, w0h, s0h), 10)
+            w0f = O.dequant_int8(w0h, s0h)
+            t_b = med(lambda: x0h @ w0f.T, 10)
+            del w0f
+            per_cfg["config0_gemv_i8row"] = {"dequant_plus_matmul_ms": round(t_a * 1e3, 2), "predequantised_matmul_ms": round(t_b * 1e3, 3),
+                                             "GBps": round(b0h / t_a * 1e-9, 3), "predequantised_GBps": round(b0h / t_b * 1e-9, 2),
+                                             "sample": "full shape, median of 10"}
+        if "cfg2" in host:
+            x2h, p2h, s2h, w8h, s8h = host["cfg2"]
+            x2b = O.f32_to_bf16(x2h)
+            x2f = O.bf16_to_f32(x2b)
+            fl = 2.0 * x2h.shape[0] * p2h.shape[0] * x2h.shape[1]
+            t_a = med(lambda: O.qgemm_int4g32_bf16(x2b, p2h, s2h), 3)
+            w2f = O.dequant_int4g32(p2h, s2h)
+            t_b = med(lambda: x2f @ w2f.T, 5)
+            del w2f
+            t_c = med(lambda: O.qgemm_int8_bf16(x2b, w8h, s8h), 3)
+            per_cfg["config2_gemm"] = {"int4_dequant_plus_matmul_ms": round(t_a * 1e3, 1), "int4_predequantised_matmul_ms": round(t_b * 1e3, 1),
+                                       "int8_dequant_plus_matmul_ms": round(t_c * 1e3, 1), "int4_TFLOPs": round(fl / t_a * 1e-12, 3),
+                                       "int4_predequantised_TFLOPs": round(fl / t_b * 1e-12, 3), "sample": "full shape, median of 3 / 5"}
+        if "cfg3" in host:
+            # one of the eight experts with the tokens routed to it; the call's time is taken as 8 x that
+            x3h, z3h, (gp, gs, up_, us_, dp, ds) = host["cfg3"]
+            idx3, _ = O.moe_route(z3h, 2, True)
+            tok0 = np.nonzero((idx3 == 0).any(axis=1))[0]
+            xe = O.f32_to_bf16(x3h[tok0])
+
+            def expert_dq():
+                g = O.qgemv_int4g32(xe, gp, gs)
+                u_ = O.qgemv_int4g32(xe, up_, us_)
+                return O.qgemv_int4g32(O.f32_to_bf16(O.silu(g) * u_), dp, ds)
+
+            t_a = med(expert_dq, 1, 0)
+            gf, uf, df = O.dequant_int4g32(gp, gs), O.dequant_int4g32(up_, us_), O.dequant_int4g32(dp, ds)
+            xef = O.bf16_to_f32(xe)
+
+            def expert_pre():
+                h = O.bf16_to_f32(O.f32_to_bf16(O.silu(xef @ gf.T) * (xef @ uf.T)))
+                return h @ df.T
+
+            t_b = med(expert_pre, 3)
+            del gf, uf, df
+            per_cfg["config3_moe_ffn"] = {"dequant_plus_matmul_ms": round(8 * t_a * 1e3, 1), "predequantised_matmul_ms": round(8 * t_b * 1e3, 1),
+                                          "sample": "expert 0 of 8 with its %d tokens, one call (three for the matmuls alone), scaled by 8" % tok0.size}
+        if "cfg4" in host:
+            # two of the 18 layers and the output table at context 2048; a token is taken as 9 x the layers + the table
+            h4 = host["cfg4"]
+            c4 = h4["cfg"]
+            ctx = 2048
+            kc = [np.zeros((ctx + 1, c4.dh), np.uint16) for _ in range(2)]
+            vc = [np.zeros((ctx + 1, c4.dh), np.uint16) for _ in range(2)]
+            xr = np.random.Generator(np.random.PCG64(1004)).standard_normal(c4.d).astype(np.float32)
+
+            def two_layers():
+                xx = xr
+                for li in range(2):
+                    xx = O.decode_layer(h4["layers"][li], xx, ctx, kc[li], vc[li], c4.hq, c4.dh, c4.eps, c4.rope_base)
+                return xx
+
+            t_l = med(two_layers, 1, 0)
+            t_t = med(lambda: O.decode_logits(h4, xr, c4.eps), 1, 0)
+            wf = [[O.dequant_int4g32(*L[k]) for k in ("wqkv", "wo", "wgu", "wd")] for L in h4["layers"]]
+            tf = O.dequant_int4g32(*h4["emb"])
+            vq, va, vh = xr, np.ones(c4.hq * c4.dh, np.float32), np.ones(c4.ffn, np.float32)
+            t_lp = med(lambda: [(wl[0] @ vq, wl[1] @ va, wl[2] @ vq, wl[3] @ vh) for wl in wf], 3)
+            t_tp = med(lambda: tf @ vq, 3)
+            del wf, tf
+            per_cfg["config4_decode_step"] = {"dequant_plus_matmul_tokens_per_s": round(1.0 / (9 * t_l + t_t), 4),
+                                              "predequantised_matmul_tokens_per_s": round(1.0 / (9 * t_lp + t_tp), 2),
+                                              "sample": "2 of 18 layers (x 9) + the 256000-row table, context 2048, one call; the matmul-only "
+                                                        "figure leaves out attention and norms"}
         cpu = {
-            "value": round(gemv_bytes(1) / med * 1e-9, 4), "unit": "GB/s", "cores": int(threads), "kind": "port",
+            "value": round(gemv_bytes(1) / t_dq * 1e-9, 4), "unit": "GB/s", "cores": int(threads), "kind": "port",
             "sample": "config 1 at M=1, full shape: numpy dequantise-to-fp32 + sgemv, median of %d calls after 1 warm-up "
-                      "(%.1f ms per call); build-written numpy baseline, no reference implementation exists in the snapshot" % (reps, med * 1e3),
-            "predequantised_sgemv_GBps": round(gemv_bytes(1) / float(np.median(t2)) * 1e-9, 3),
-            "host_cpus": os.cpu_count(),
+                      "(%.1f ms per call); build-written numpy baseline, no reference implementation exists in the snapshot" % (reps, t_dq * 1e3),
+            "predequantised_sgemv_GBps": round(gemv_bytes(1) / t_pre * 1e-9, 3),
+            "host_cpus": os.cpu_count(), "blas_threads": int(threads), "oracle_dequant_workers": int(O.WORKERS),
+            "configs": per_cfg,
         }
 
     traffic_bytes, kernel_name = profile_figures()
@@ -450,6 +560,8 @@ def main():
                    "algorithmic_bytes_per_launch": gemv_bytes(1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_bytes,
+                     "traffic_source": "hardware counters of an earlier profiled run, read from the committed summary "
+                                       "profiles/gemv_i4g32_m1_config1_hbm_traffic.txt (not measured by this run)",
                      "kernel": kernel_name, "wall_clock_us_per_step": round(wall1, 3)},
         "cpu_baseline": cpu,
         "parity": parity,

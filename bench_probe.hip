@@ -38,3 +38,12 @@ extern "C" int bench_probe_read(const void *src, int64_t bytes, uint32_t *out, v
                        reinterpret_cast<const uint8_t *>(src), nwaves, out);
     return (int)hipGetLastError();
 }
+
+// A kernel that does nothing (one workgroup of one wave): what a dependent launch costs in a replayed graph on this
+// machine, the floor under every small kernel of the decode step.
+__global__ void probe_empty_kernel() {}
+
+extern "C" int bench_probe_empty(void *stream) {
+    hipLaunchKernelGGL(probe_empty_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream);
+    return (int)hipGetLastError();
+}

@@ -45,7 +45,7 @@ int dequant_i4g32_launch(const uint8_t *, const uint16_t *, float *, int, int, h
 int dequant_i8row_launch(const int8_t *, const float *, float *, int, int, hipStream_t);
 int gemv_i4g32_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
 int gemv_i4g32_mfma_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, int, hipStream_t);
-int gemv_i8row_dispatch(const float *, const int8_t *, const float *, float *, int, int, int, hipStream_t);
+int gemv_i8row_dispatch(const float *, const int8_t *, const float *, float *, int, int, int, bool, hipStream_t);
 int gemm_i4g32_bf16_dispatch(const uint16_t *, const uint8_t *, const uint16_t *, uint16_t *, int, int, int,
                              hipStream_t);
 int gemm_i8row_bf16_dispatch(const uint16_t *, const int8_t *, const float *, uint16_t *, int, int, int,
@@ -203,15 +203,26 @@ int chadq_gemv_i4g32_addnorm_geglu(const float *res, const float *delta, int n_d
     return gemv_i4g32_addnorm_geglu_launch(res, delta, delta ? n_delta : 0, norm_w, eps, res_out, wp, scale_f16, h_bf16, N, K, st);
 }
 
+static int gemv_i8row_entry(const char *name, bool fp32_only, const float *x, const int8_t *w8, const float *scale, float *y, int M,
+                           int N, int K, hipStream_t st) {
+    CHADQ_REQUIRE(M >= 1 && M <= 16, CHADQ_ERR_SHAPE, "%s: M=%d outside [1,16]", name, M);
+    CHADQ_REQUIRE(N >= 0 && K >= 16 && K % 16 == 0, CHADQ_ERR_SHAPE, "%s: N=%d K=%d (K must be a positive multiple of 16)", name, N, K);
+    if (N == 0) return 0;
+    CHADQ_REQUIRE(x && w8 && scale && y, CHADQ_ERR_NULL, "%s: null pointer", name);
+    CHADQ_REQUIRE(aligned16(x) && aligned16(w8), CHADQ_ERR_ALIGN, "%s: x and w8 must be 16-byte aligned", name);
+    return gemv_i8row_dispatch(x, w8, scale, y, M, N, K, fp32_only, st);
+}
+
 int chadq_gemv_i8row(const float *x, const int8_t *w8, const float *scale, float *y, int M, int N, int K,
                      void *stream) {
     ENTER();
-    CHADQ_REQUIRE(M >= 1 && M <= 16, CHADQ_ERR_SHAPE, "chadq_gemv_i8row: M=%d outside [1,16]", M);
-    CHADQ_REQUIRE(N >= 0 && K >= 16 && K % 16 == 0, CHADQ_ERR_SHAPE, "chadq_gemv_i8row: N=%d K=%d (K must be a positive multiple of 16)", N, K);
-    if (N == 0) return 0;
-    CHADQ_REQUIRE(x && w8 && scale && y, CHADQ_ERR_NULL, "chadq_gemv_i8row: null pointer");
-    CHADQ_REQUIRE(aligned16(x) && aligned16(w8), CHADQ_ERR_ALIGN, "chadq_gemv_i8row: x and w8 must be 16-byte aligned");
-    return gemv_i8row_dispatch(x, w8, scale, y, M, N, K, st);
+    return gemv_i8row_entry("chadq_gemv_i8row", false, x, w8, scale, y, M, N, K, st);
+}
+
+int chadq_gemv_i8row_fp32(const float *x, const int8_t *w8, const float *scale, float *y, int M, int N, int K,
+                          void *stream) {
+    ENTER();
+    return gemv_i8row_entry("chadq_gemv_i8row_fp32", true, x, w8, scale, y, M, N, K, st);
 }
 
 int chadq_gemm_i4g32_bf16(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *scale_f16, uint16_t *y_bf16,

@@ -2,14 +2,15 @@
 //
 // HBM-bound stream of W.  A wavefront owns whole rows; one 128-bit load per lane = 16 weights, a wave-wide
 // load = 1024 consecutive k (1 KiB contiguous).  All loads of a wave are issued first; the fp32 activations
-// come once per workgroup, through LDS, and a lane's k positions stay in registers.  Signed bytes are flipped to unsigned
-// (w ^ 0x80 = w + 128) so that v_cvt_f32_ubyteN converts them in one instruction; the accumulator starts
-// at -128 * sum(x) to take the offset back out.  DPP adds fold the 64 partial sums; no LDS.
+// come once per workgroup, through LDS, and a lane's k positions stay in registers.  A signed byte becomes a float in one
+// instruction (v_cvt_f32_i32 with a sign-extending byte select), so every product is x[k] * float(W[n,k]) itself: an
+// activation's error does not depend on its neighbours (flipping the bytes to unsigned for v_cvt_f32_ubyteN and taking
+// 128 * sum(x) back out costs the same and does depend on them).  DPP adds fold the 64 partial sums; no LDS.
 #include "chadq_common.h"
 
 namespace chadq {
 
-__device__ __forceinline__ float ubyte_to_f32(uint32_t v, int i) { return (float)((v >> (8 * i)) & 0xFFu); }
+__device__ __forceinline__ float sbyte_to_f32(uint32_t v, int i) { return (float)(int)(int8_t)(v >> (8 * i)); }
 
 template <int CH, int R, int MB, int WPB>
 __global__ __launch_bounds__(64 * WPB) void gemv_i8row_rows_kernel(const float *__restrict__ x,
@@ -59,10 +60,8 @@ __global__ __launch_bounds__(64 * WPB) void gemv_i8row_rows_kernel(const float *
         }
     __syncthreads();
     float xs[MB][CH][16];
-    float bias[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) {
-        float sum = 0.f;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
 #pragma unroll
@@ -73,26 +72,23 @@ __global__ __launch_bounds__(64 * WPB) void gemv_i8row_rows_kernel(const float *
                 xs[m][c][4 * i + 1] = v.y;
                 xs[m][c][4 * i + 2] = v.z;
                 xs[m][c][4 * i + 3] = v.w;
-                sum += (v.x + v.y) + (v.z + v.w);
             }
         }
-        bias[m] = -128.f * sum;
     }
 
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         float acc[MB];
 #pragma unroll
-        for (int m = 0; m < MB; ++m) acc[m] = bias[m];
+        for (int m = 0; m < MB; ++m) acc[m] = 0.f;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
-            const uint32_t ww[4] = {w[r][c].x ^ 0x80808080u, w[r][c].y ^ 0x80808080u, w[r][c].z ^ 0x80808080u,
-                                    w[r][c].w ^ 0x80808080u};
+            const uint32_t ww[4] = {w[r][c].x, w[r][c].y, w[r][c].z, w[r][c].w};
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const float f = ubyte_to_f32(ww[j], i);
+                    const float f = sbyte_to_f32(ww[j], i);
 #pragma unroll
                     for (int m = 0; m < MB; ++m) acc[m] = __builtin_fmaf(xs[m][c][4 * j + i], f, acc[m]);
                 }
@@ -120,15 +116,15 @@ __global__ __launch_bounds__(256) void gemv_i8row_generic_kernel(const float *__
         float acc = 0.f;
         for (int k0 = lane * 16; k0 < K; k0 += 1024) {
             const u32x4 wv = *reinterpret_cast<const u32x4 *>(w8 + (size_t)row * K + k0);
-            const uint32_t ww[4] = {wv.x ^ 0x80808080u, wv.y ^ 0x80808080u, wv.z ^ 0x80808080u, wv.w ^ 0x80808080u};
+            const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
             const f32x4 *xp = reinterpret_cast<const f32x4 *>(x + (size_t)m * K + k0);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const f32x4 v = xp[j];
-                acc = __builtin_fmaf(v.x, ubyte_to_f32(ww[j], 0) - 128.f, acc);
-                acc = __builtin_fmaf(v.y, ubyte_to_f32(ww[j], 1) - 128.f, acc);
-                acc = __builtin_fmaf(v.z, ubyte_to_f32(ww[j], 2) - 128.f, acc);
-                acc = __builtin_fmaf(v.w, ubyte_to_f32(ww[j], 3) - 128.f, acc);
+                acc = __builtin_fmaf(v.x, sbyte_to_f32(ww[j], 0), acc);
+                acc = __builtin_fmaf(v.y, sbyte_to_f32(ww[j], 1), acc);
+                acc = __builtin_fmaf(v.z, sbyte_to_f32(ww[j], 2), acc);
+                acc = __builtin_fmaf(v.w, sbyte_to_f32(ww[j], 3), acc);
             }
         }
         const float t = wave_sum_to_lane63(acc);
@@ -146,11 +142,12 @@ static void launch_rows8(const float *x, const int8_t *w8, const float *sc, floa
 bool gemv_i8row_mfma_ok(int M, int K);
 int gemv_i8row_mfma_launch(const float *, const int8_t *, const float *, float *, int, int, int, hipStream_t);
 
-int gemv_i8row_dispatch(const float *x, const int8_t *w8, const float *sc, float *y, int M, int N, int K,
+// fp32_only: the fp32 kernels for every K (chadq_gemv_i8row_fp32)
+int gemv_i8row_dispatch(const float *x, const int8_t *w8, const float *sc, float *y, int M, int N, int K, bool fp32_only,
                         hipStream_t st) {
     // K a multiple of 128: the int8 matrix core, one pass over W for all M (gemv_i8row_mfma.hip); the fp32 kernels
     // below keep the other row lengths
-    if (N > 0 && gemv_i8row_mfma_ok(M, K)) return gemv_i8row_mfma_launch(x, w8, sc, y, M, N, K, st);
+    if (!fp32_only && N > 0 && gemv_i8row_mfma_ok(M, K)) return gemv_i8row_mfma_launch(x, w8, sc, y, M, N, K, st);
     // <1024-wide chunks per row, rows per wave, activation rows, waves per workgroup>, picked by measurement: eight
     // waves share one copy of the activations; matrices with many rows give a wave 2 or 4 rows
     if (K <= 2048) {

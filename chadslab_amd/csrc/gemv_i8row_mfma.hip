@@ -6,9 +6,13 @@
 // with a power-of-two scale, X = rint(x * 2^(20 - e)) with 2^e <= max|x| < 2^(e+1) (|X| <= 2^21), and X as three
 // balanced base-256 digits, X = a0 * 2^16 + a1 * 2^8 + a2 with -128 <= a <= 127.  Each digit is one int8 operand
 // row; the three int32 dot products are exact and meet again in fp32: y = s[n] * sum over blocks 2^(e-20) * (D0 *
-// 2^16 + D1 * 2^8 + D2).  What is dropped is below 2^-22 of the block's largest |x| per element (the result is held
-// to a 1e-3 relative tolerance); integer-valued activations below 2^20 are represented exactly, so their sums are
-// exact integers as in the per-row kernel.  A block with a non-finite activation makes its rows' results NaN.
+// 2^16 + D1 * 2^8 + D2).  What is dropped is at most 2^-21 of the block's largest |x| per element, so a result is off by
+// at most scale[n] * sum over blocks of 2^-21 * max_block|x| * sum_{k in block} |W[n,k]| (the result is held to a 1e-3
+// relative tolerance; one outlier among the activations costs the small elements of its block their low bits, also
+// in rows whose weight at the outlier is zero: chadq_gemv_i8row_fp32 is the form without this).  Integer-valued
+// activations below 2^20 are represented exactly and the three digit sums are recombined exactly (in float64), so
+// integer sums below 2^24 are exact as in the per-row kernel.  A block with a non-finite activation makes its rows'
+// results NaN (the fp32 kernels follow IEEE arithmetic element by element).
 //
 // One MFMA, D[16x16] += A[16x64] * B[64x16]:
 //   B = weights.  Column c is weight row n0 + c (16 rows per wave); lane (c, g = lane/16) supplies 16 k-slots.  A
@@ -222,18 +226,23 @@ __global__ __launch_bounds__(512) void gemv_i8row_mfma_kernel(const float *__res
                     acc[s][jj] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, jj ? b1 : b0, acc[s][jj], 0, 0, 0);
                 }
         }
-        // the block's digit sums -> fp32 with the block's scales
+        // the block's digit sums -> fp32 with the block's scales.  D0 * 2^16 + D1 * 2^8 + D2 can need more than the 24
+        // bits of a float before its terms cancel, so the three are combined in float64 (exact: below 2^53) and rounded
+        // to fp32 once
+        auto combine = [](int d0, int d1, int d2) {
+            return (float)__builtin_fma((double)d0, 65536.0, __builtin_fma((double)d1, 256.0, (double)d2));
+        };
         if constexpr (SETS == 3) {
             const i32x4 e0 = acc[0][0] + acc[0][1], e1 = acc[1][0] + acc[1][1], e2 = acc[2][0] + acc[2][1];
             const int q0[4] = {e0.x, e0.y, e0.z, e0.w}, q1[4] = {e1.x, e1.y, e1.z, e1.w}, q2[4] = {e2.x, e2.y, e2.z, e2.w};
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                yacc[r] = __builtin_fmaf(bscale[r], __builtin_fmaf((float)q0[r], 65536.f, __builtin_fmaf((float)q1[r], 256.f, (float)q2[r])), yacc[r]);
+                yacc[r] = __builtin_fmaf(bscale[r], combine(q0[r], q1[r], q2[r]), yacc[r]);
         } else {
 #pragma unroll
             for (int s = 0; s < SETS; ++s) {
                 const i32x4 e = acc[s][0] + acc[s][1];
-                yacc[s] = __builtin_fmaf(bscale[s], __builtin_fmaf((float)e.x, 65536.f, __builtin_fmaf((float)e.y, 256.f, (float)e.z)), yacc[s]);
+                yacc[s] = __builtin_fmaf(bscale[s], combine(e.x, e.y, e.z), yacc[s]);
             }
         }
     };

@@ -76,12 +76,18 @@ def dequantize(qw: QWeight) -> torch.Tensor:
     raise TypeError("unknown weight container %r" % type(qw))
 
 
-def qgemv(x: torch.Tensor, qw: QWeight, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Decode product, fp32 out [M,N], M <= 16.  x is bf16 [M,K] for int4 weights, fp32 [M,K] for int8 weights."""
+def qgemv(x: torch.Tensor, qw: QWeight, out: Optional[torch.Tensor] = None, *, fp32_elements: bool = False) -> torch.Tensor:
+    """Decode product, fp32 out [M,N], M <= 16.  x is bf16 [M,K] for int4 weights, fp32 [M,K] for int8 weights.
+
+    fp32_elements (int8 weights only): fp32 arithmetic on every activation (chadq_gemv_i8row_fp32) instead of the
+    matrix-core kernel's per-block fixed point, whose error on a small activation grows with the largest one of its
+    2048-k block; the weights are then streamed once per pair of activation rows."""
     lib = _lib.load()
     if x.dim() != 2 or x.shape[1] != qw.K:
         raise ValueError("x must be [M,%d], got %s" % (qw.K, tuple(x.shape)))
     m = x.shape[0]
+    if fp32_elements and not isinstance(qw, QWeightInt8):
+        raise ValueError("fp32_elements applies to int8 weights (fp32 activations) only")
     if isinstance(qw, QWeightInt4G32):
         x = _dev(x, "x", torch.bfloat16)
         p, s = _dev(qw.packed, "packed", torch.uint8), _dev(qw.scale, "scale", torch.float16)
@@ -93,8 +99,8 @@ def qgemv(x: torch.Tensor, qw: QWeight, out: Optional[torch.Tensor] = None) -> t
         x = _dev(x, "x", torch.float32)
         w, s = _dev(qw.w, "w", torch.int8), _dev(qw.scale, "scale", torch.float32)
         y = _out(out, (m, qw.N), torch.float32, x.device)
-        _lib.check(lib.chadq_gemv_i8row(x.data_ptr(), w.data_ptr(), s.data_ptr(), y.data_ptr(), m, qw.N, qw.K,
-                                        _stream()), "chadq_gemv_i8row")
+        fn, name = (lib.chadq_gemv_i8row_fp32, "chadq_gemv_i8row_fp32") if fp32_elements else (lib.chadq_gemv_i8row, "chadq_gemv_i8row")
+        _lib.check(fn(x.data_ptr(), w.data_ptr(), s.data_ptr(), y.data_ptr(), m, qw.N, qw.K, _stream()), name)
         return y
     raise TypeError("unknown weight container %r" % type(qw))
 

@@ -120,13 +120,26 @@ int chadq_gemv_i4g32_addnorm_geglu(const float *res, const float *delta, int n_d
 /*
  * y[m,n] = scale[n] * sum_k x[m,k] * W[n,k]                                 (config 0)
  * x fp32 [M,K], W int8 [N,K], scale fp32 [N], y fp32 [M,N], 1 <= M <= 16, K % 16 == 0.
- * K % 128 == 0: the weights are read once for all M rows, on the int8 matrix core; per activation row and 2048 k the
- * activations are held as three 8-bit fixed-point digits with a power-of-two scale (dropped: < 2^-22 of the block's
- * largest |x| per element; integer activations below 2^20 stay exact; a non-finite activation makes its row NaN), and
- * a row's result does not depend on M.  Other K: fp32 arithmetic, the weights streamed once per pair of activation rows.
+ * K % 128 == 0: the weights are read once for all M rows, on the int8 matrix core; per activation row and block of
+ * 2048 k the activations are held in fixed point (three 8-bit digits, a power-of-two scale from the block's largest
+ * |x|), the integer sums are exact.  Bound: |y[m,n] - exact| <= |scale[n]| * sum over blocks b of
+ * 2^-21 * max_{k in b}|x[m,k]| * sum_{k in b}|W[n,k]| (+ the fp32 rounding of the block sums).  For activations of one
+ * order of magnitude that is 1e-6 relative; ONE outlier in a block costs the block's small elements their low bits,
+ * also in output rows whose weight at the outlier is zero - call chadq_gemv_i8row_fp32 where that matters.  Integer
+ * activations below 2^20 whose sums stay below 2^24 give exact results; a non-finite activation makes its row NaN;
+ * a row's result does not depend on M.  Other K: fp32 arithmetic as in chadq_gemv_i8row_fp32.
  */
 int chadq_gemv_i8row(const float *x, const int8_t *w8, const float *scale, float *y, int M, int N, int K,
                      void *stream);
+
+/*
+ * The same product with fp32 arithmetic on every element, whatever K: x[m,k] * float(W[n,k]) accumulated in fp32, the
+ * row scale applied to the sum; the weights are streamed once per pair of activation rows (M = 1, 2: the speed of
+ * chadq_gemv_i8row within a few per cent; M = 8: four passes).  Same argument rules.  An activation's error does not
+ * depend on its neighbours; non-finite activations behave as IEEE arithmetic has them (inf * W is an infinity, inf * 0 a NaN).
+ */
+int chadq_gemv_i8row_fp32(const float *x, const int8_t *w8, const float *scale, float *y, int M, int N, int K,
+                          void *stream);
 
 /* ---- prefill dequant-GEMM (benchmark config 2) ---------------------------------------- */
 

@@ -584,7 +584,8 @@ def test_decoder_step_config4_full_size_graph_replay():
 
     An 18-layer random-weight network amplifies rounding differences: two CPU restatements that differ only in the
     precision of the GEMV sums (fp32 against float64, same bf16 rounding points) end 8.8e-3 apart in the logits
-    (2.0e-3 after two layers), so an end-to-end bound of 1e-2 separates nothing at this depth.  The check is
+    (2.0e-3 after two layers; tests/test_decode_rounding_growth.py reproduces both figures on the CPU), so an end-to-end
+    bound of 1e-2 separates nothing at this depth.  The check is
     therefore made where it is sharp: every layer of the GPU step is compared with the oracle's layer applied to the
     same input (the residual vector the GPU step itself had there), the logits with the oracle's output projection of
     the GPU's final residual vector; the graph-replayed step must then reproduce the eager one bit for bit; the
@@ -655,16 +656,16 @@ def test_decoder_step_config4_full_size_graph_replay():
     want = O.decode_step(m, tok, pos0, kc2, vc2, cfg.hq, cfg.dh, cfg.eps, cfg.rope_base)
     e2e = O.rel_l2(eager_logits, want)
     print("end-to-end rel-L2 of the logits against the oracle's own 18-layer step: %.3e" % e2e, flush=True)
-    assert e2e < 5e-2
+    assert e2e < 2e-2   # measured 1.4e-2; two CPU restatements differ by 8.8e-3 here (tests/test_decode_rounding_growth.py)
     top2 = np.sort(want)[-2:]
-    if top2[1] - top2[0] > 5e-2 * np.abs(want).max():
+    if top2[1] - top2[0] > 2.0 * np.abs(eager_logits - want).max():  # the oracle's winner leads by more than the logits differ
         assert eager_tok == int(np.argmax(want))
     dec.graph.replay()  # position 2048 with the token the first step chose
     torch.cuda.synchronize()
     want2 = O.decode_step(m, eager_tok, pos0 + 1, kc2, vc2, cfg.hq, cfg.dh, cfg.eps, cfg.rope_base)
     got2 = dec.logits.cpu().numpy()
     assert int(dec.pos.item()) == pos0 + 2 and np.isfinite(got2).all()
-    assert O.rel_l2(got2, want2) < 5e-2, "second step: %.3e" % O.rel_l2(got2, want2)
+    assert O.rel_l2(got2, want2) < 2.5e-2, "second step: %.3e" % O.rel_l2(got2, want2)
 
 
 def test_decoder_refuses_positions_past_the_cache_and_tokens_outside_the_table():

@@ -291,6 +291,86 @@ def test_gemv_int8_outliers_zero_rows_and_non_finite_values(ops):
     assert np.array_equal(y2[:4], y[:4])                      # ... and no other
 
 
+def test_gemv_int8_outlier_column_error_bound_per_element(ops):
+    """The matrix-core int8 GEMV holds a block of 2048 activations in fixed point relative to the block's largest |x|:
+    the header's bound |err| <= |s[n]| * sum over blocks of 2^-21 * max|x| * sum|W[n,k]| is checked element by element
+    with one outlier column, in particular on output rows whose weight at the outlier is ZERO (there the outlier adds
+    nothing to the exact result and the whole difference is the other elements' lost low bits).  chadq_gemv_i8row_fp32
+    has no such term: the same inputs come out at fp32 accuracy."""
+    m_rows, n, k = 5, 512, 4096
+    x, w, s, _ = i8_case(781, m_rows, n, k)
+    col = 17
+    x[:, col] = 3.0e6 * np.array([1, -1, 1, 1, -1], np.float32)
+    w[::2, col] = 0                              # every other output row ignores the outlier
+    x[3, 2048 + 5] = -7.0e4                      # a second, smaller outlier in row 3's second block
+    from chadslab_amd import QWeightInt8
+
+    q8 = QWeightInt8(torch.from_numpy(w).to(DEV), torch.from_numpy(s).to(DEV))
+    xt = torch.from_numpy(x).to(DEV)
+    ref = O.qgemv_int8_f64(x, w, s)
+    y = ops.qgemv(xt, q8).cpu().numpy().astype(np.float64)
+    aw = np.abs(w.astype(np.float64))
+    bound = np.zeros((m_rows, n))
+    for b0 in range(0, k, 2048):
+        bmax = np.abs(x[:, b0:b0 + 2048]).max(axis=1).astype(np.float64)            # [M]
+        bound += 2.0 ** -21 * bmax[:, None] * aw[:, b0:b0 + 2048].sum(axis=1)[None, :]
+    bound = np.abs(s.astype(np.float64))[None, :] * bound
+    slack = 4e-7 * np.abs(ref) + 1e-30                                               # the fp32 roundings of the sums
+    err = np.abs(y - ref)
+    assert (err <= bound + slack).all(), float((err / (bound + slack)).max())
+    # the bound is not vacuous: on the rows that ignore the outlier the error is a visible fraction of the result ...
+    zero_rows = err[:, ::2] / (np.abs(ref[:, ::2]) + 1e-30)
+    assert np.median(zero_rows) > 1e-3
+    # ... and the fp32 form has none of it
+    yf = ops.qgemv(xt, q8, fp32_elements=True).cpu().numpy().astype(np.float64)
+    mag = (np.abs(x.astype(np.float64)) @ (aw * np.abs(s.astype(np.float64))[:, None]).T)  # sum of |terms|
+    assert (np.abs(yf - ref) <= 1e-5 * mag).all()
+    assert np.median(np.abs(yf[:, ::2] - ref[:, ::2]) / (np.abs(ref[:, ::2]) + 1e-30)) < 1e-5
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 16384, 2048), (2, 300, 4096), (5, 333, 2048), (16, 70, 6144), (3, 100, 1040)])
+def test_gemv_int8_fp32_elements_entry_point(ops, m, n, k):
+    x, w, s, q8 = i8_case(790 + m, m, n, k)
+    y = ops.qgemv(torch.from_numpy(x).to(DEV), q8, fp32_elements=True).cpu().numpy()
+    assert O.rel_l2(y, O.qgemv_int8_f64(x, w, s)) <= TOL_F32
+    xi = rng(791 + m).integers(-2000, 2001, (m, k)).astype(np.float32)
+    one = type(q8)(q8.w, torch.ones_like(q8.scale))
+    yi = ops.qgemv(torch.from_numpy(xi).to(DEV), one, fp32_elements=True).cpu().numpy()
+    want = xi.astype(np.int64) @ w.astype(np.int64).T
+    ok = np.abs(want) < 2 ** 24
+    assert np.array_equal(yi[ok].astype(np.int64), want[ok])
+    xinf = x.copy()
+    xinf[0, 3] = np.inf
+    yinf = ops.qgemv(torch.from_numpy(xinf).to(DEV), q8, fp32_elements=True).cpu().numpy()
+    nz = w[:, 3] != 0  # IEEE arithmetic element by element: inf * w is an infinity, inf * 0 a NaN
+    assert np.isinf(yinf[0][nz]).all() and np.isnan(yinf[0][~nz]).all()
+    assert np.isfinite(yinf[1:]).all()
+
+
+def test_gemv_int8_integer_digit_sums_that_cancel_stay_exact(ops):
+    """The matrix-core kernel sums three base-256 digits of the fixed-point activations separately and recombines
+    D0 * 2^16 + D1 * 2^8 + D2.  Here the digit sums are far beyond 2^24 and cancel: x = 32768 (digits 1, -128, 0)
+    against weights +64 and x = 32512 (digits 0, 127, 0) against weights -64, so D0 * 2^16 = 2.1e9 and D1 * 2^8 = -2.1e9
+    while the result is 8.4e6 + small.  Recombined in float64 the result is the exact integer (fp32 recombination
+    was off by up to 128 here)."""
+    n, k = 64, 2048
+    r = rng(795)
+    w = np.zeros((n, k), np.int8)
+    x = np.zeros((1, k), np.float32)
+    x[0, 0:1024:2], x[0, 1:1024:2] = 32768.0, 32512.0
+    w[:, 0:1024:2], w[:, 1:1024:2] = 64, -64
+    w[:, 0:1024:2] += r.integers(-1, 2, (n, 512)).astype(np.int8)   # a little variety per output row
+    x[0, 1024:1100] = r.integers(-50, 51, 76)                        # the other half of K: small integers
+    w[:, 1024:1100] = r.integers(-127, 128, (n, 76))
+    from chadslab_amd import QWeightInt8
+
+    q8 = QWeightInt8(torch.from_numpy(w).to(DEV), torch.ones(n, device=DEV))
+    want = x.astype(np.int64) @ w.astype(np.int64).T
+    assert np.abs(want).max() < 2 ** 24 and np.abs(want).min() > 2 ** 22
+    y = ops.qgemv(torch.from_numpy(x).to(DEV), q8).cpu().numpy()
+    assert np.array_equal(y.astype(np.int64), want)
+
+
 # ------------------------------------------------------------------ seeded random shapes (ragged edges of every kind)
 def test_random_shapes_int4_gemv_and_gemm(ops):
     r = rng(4242)
