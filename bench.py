@@ -59,7 +59,8 @@ def parse():
     ap.add_argument("--no-extras", action="store_true", help="skip the side measurements")
     ap.add_argument("--extras", default="gemv,int8,gemm,moe,decode",
                     help="comma list of the side measurements to run (gemv, int8, gemm, moe, decode; moe_ablation adds, "
-                         "to moe, the tile-order call on the two measurement builds of the expert GEMM)")
+                         "to moe, the tile-order call on the two measurement builds of the expert GEMM; gemm_ablation "
+                         "adds, to gemm, config 2 on the build without dequantisation)")
     ap.add_argument("--short", action="store_true",
                     help="few launches per side measurement: for hardware-counter runs, which serialise every dispatch")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -239,7 +240,7 @@ def main():
             bm = N0 * K0 + N0 * 4 + m * (K0 * 4 + N0 * 4)
             extras["gemv_i8row_config0"][f"M{m}_extra"] = {"us": round(usm, 3), "GBps": round(bm / usm * 1e-3, 1)}
         del c0, w0
-    if "gemm" in want:
+    if "gemm" in want or "gemm_ablation" in want:
         # config 2: prefill dequant-GEMM, int4 group-32 and int8 per-row
         M2, N2, K2 = 512, 4096, 4096
         r2 = np.random.Generator(np.random.PCG64(1002))
@@ -258,6 +259,20 @@ def main():
             extras[name] = {"us": round(usg, 3), "TFLOPs": round(flop / usg * 1e-6, 1),
                             "frac_bf16_mfma_peak": round(flop / usg * 1e-6 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
+        if "gemm_ablation" in want:
+            # the same two calls on the measurement build whose 128 x 64 kernel hands the packed words to the matrix
+            # core without dequantising them: the floor under any variant of that kernel with cheaper (or no)
+            # dequantisation, e.g. int8 weights on the int8 matrix core
+            from chadslab_amd.build import ablation_path
+
+            main_lib = _lib.load()
+            if ablation_path("nodequant").exists():
+                try:
+                    _lib._lib = _lib.open_library(ablation_path("nodequant"))
+                    for name, qw in (("gemm_i4g32_config2", q4), ("gemm_i8row_config2", q8)):
+                        extras[name]["us_without_dequantisation"] = round(run_steps(lambda i: ops.qgemm(x2, qw, out=y2), *n_gemm)[0], 3)
+                finally:
+                    _lib._lib = main_lib
         # context: the vendor library's plain bf16 GEMM (no dequantisation) on the same shape, through torch.matmul
         wb16 = torch.randn(N2, K2, device=dev).to(torch.bfloat16)
         yt = torch.empty(M2, N2, dtype=torch.bfloat16, device=dev)
@@ -346,7 +361,7 @@ def main():
             main_lib = _lib.load()
             abl = {"both": extras["moe_ffn_i4g32_config3_tiled"]["us"]}
             try:
-                for name in ABLATIONS:
+                for name in ("stream", "arith"):
                     if not ablation_path(name).exists():
                         abl[name] = None
                         continue

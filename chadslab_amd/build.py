@@ -59,14 +59,16 @@ def build(verbose: bool = True, save_temps: bool = False) -> Path:
     os.replace(tmp, LIB)
     if verbose:
         print("built %s (%d sources)" % (LIB, len(srcs)))
+    build_ablations(verbose)  # always together: the measurement builds share every other object and the whole C ABI
     return LIB
 
 
-# Measurement builds of the tile-order expert GEMM (bench.py --extras moe_ablation): the same library with one half of
-# that kernel's loop compiled out, so that each half's share of the time can be measured on its own.  Their results are
-# wrong by construction; nothing but the bench loads them.
-ABLATIONS = {"stream": 1,  # memory traffic without arithmetic
-             "arith": 2}   # arithmetic without weight loads
+# Measurement builds (bench.py --extras moe_ablation / gemm_ablation): the same library with a part of one kernel's loop
+# compiled out, so that the part's share of the time can be measured on its own.  Their results are wrong by
+# construction; nothing but the bench loads them.  name -> (source file, macro definition)
+ABLATIONS = {"stream": ("gemm_expert_i4g32.hip", "-DCHADQ_EXPERT_ABLATE=1"),   # expert GEMM: memory traffic without arithmetic
+             "arith": ("gemm_expert_i4g32.hip", "-DCHADQ_EXPERT_ABLATE=2"),    # expert GEMM: arithmetic without weight loads
+             "nodequant": ("gemm_q_bf16.hip", "-DCHADQ_GEMM_ABLATE=1")}        # prefill GEMM (128 x 64 tile): no dequantisation
 
 
 def ablation_path(name: str) -> Path:
@@ -74,13 +76,19 @@ def ablation_path(name: str) -> Path:
 
 
 def build_ablations(verbose: bool = True) -> None:
-    """Needs build() to have run: only gemm_expert_i4g32.hip is recompiled, the other objects are shared."""
-    src = CSRC / "gemm_expert_i4g32.hip"
-    others = [o for o in sorted(OBJ.glob("*.o")) if o.stem != src.stem and not o.stem.startswith("ablate_") and
-              (CSRC / (o.stem + ".hip")).exists()]
-    for name, mode in ABLATIONS.items():
+    """Only the one source file of each ablation is recompiled; the other objects are those of the library."""
+    def one(item):
+        name, (fname, define) = item
+        src = CSRC / fname
         obj = OBJ / ("ablate_%s.o" % name)
-        _run([HIPCC, *FLAGS, "-DCHADQ_EXPERT_ABLATE=%d" % mode, "-c", str(src), "-o", str(obj)])
+        _run([HIPCC, *FLAGS, define, "-c", str(src), "-o", str(obj)])
+        return name, src, obj
+
+    with ThreadPoolExecutor(max_workers=len(ABLATIONS)) as ex:
+        done = list(ex.map(one, ABLATIONS.items()))
+    for name, src, obj in done:
+        others = [o for o in sorted(OBJ.glob("*.o")) if o.stem != src.stem and not o.stem.startswith("ablate_") and
+                  (CSRC / (o.stem + ".hip")).exists()]
         tmp = ablation_path(name).with_suffix(".so.tmp")
         _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, others), str(obj)])
         os.replace(tmp, ablation_path(name))
@@ -90,5 +98,3 @@ def build_ablations(verbose: bool = True) -> None:
 
 if __name__ == "__main__":
     build(save_temps="--save-temps" in sys.argv)
-    if "--ablations" in sys.argv:
-        build_ablations()

@@ -25,6 +25,8 @@ int hip_check(hipError_t e, const char *what) {
     return fail(CHADQ_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
+int attn_mqa_fused_static_init(int dev);
+
 int check_device() {
     static int ok_mask[64] = {0};  // 0 unknown, 1 ok, -1 wrong arch; benign race: idempotent values
     int dev = 0;
@@ -33,8 +35,16 @@ int check_device() {
     hipDeviceProp_t prop;
     CHADQ_HIP(hipGetDeviceProperties(&prop, dev));
     const bool ok = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
-    if (dev >= 0 && dev < 64) ok_mask[dev] = ok ? 1 : -1;
-    if (!ok) return fail(CHADQ_ERR_DEVICE, "device %d is %s; libchadq is built for gfx950 only", dev, prop.gcnArchName);
+    if (!ok) {
+        if (dev >= 0 && dev < 64) ok_mask[dev] = -1;
+        return fail(CHADQ_ERR_DEVICE, "device %d is %s; libchadq is built for gfx950 only", dev, prop.gcnArchName);
+    }
+    // first entry-point call on this device: look up the address of the attention scratch array now, so that
+    // chadq_attn_decode_mqa_fused_static itself never has to (it may be called under graph capture, where the lookup
+    // is not allowed)
+    int rc = attn_mqa_fused_static_init(dev);
+    if (rc != 0) return rc;
+    if (dev >= 0 && dev < 64) ok_mask[dev] = 1;
     return 0;
 }
 

@@ -688,7 +688,8 @@ int attn_mqa_fused_launch(const float *qkv, const int32_t *pos, const float *tab
 // The split-context partials (32 positions per slice: running maximum, sum and dh weighted columns per head) go to a
 // file-scope device array instead: 256 slices (a cache of up to 8192 rows) x 8 heads x (256 + 2) floats = 2,113,536
 // bytes, held by every GPU the library runs on until the process ends.  In host code the array's name is only a
-// stand-in for the symbol; its address on a device comes from hipGetSymbolAddress, asked once per device and kept.
+// stand-in for the symbol; its address on a device comes from hipGetSymbolAddress, asked once per device - by the first
+// call of any entry point on that device, so never under graph capture - and kept.
 // Nothing in the array has to start at zero: a call writes the slices 0 .. pos/32 before the combine kernel reads
 // exactly those.  Calls that overlap on one GPU (two streams) would share the array and race.
 constexpr int ATT_STATIC_MAX_CTX = 8192;
@@ -698,17 +699,24 @@ static std::atomic<float *> g_scratch_ptr[64];  // per device; zero-initialised
 
 int attn_mqa_fused_static_max_ctx() { return ATT_STATIC_MAX_CTX; }
 
+// Called once per device, from the first entry-point call made on it (api.hip, check_device), with that device current.
+int attn_mqa_fused_static_init(int dev) {
+    if (dev < 0 || dev >= 64) return 0;  // such a device gets no scratch; the entry point refuses it
+    if (g_scratch_ptr[dev].load(std::memory_order_acquire)) return 0;
+    float *ptr = nullptr;
+    CHADQ_HIP(hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)));
+    CHADQ_REQUIRE(ptr != nullptr, CHADQ_ERR_HIP, "hipGetSymbolAddress returned a null address for the attention scratch");
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // two threads racing here obtain the same address
+    return 0;
+}
+
 int attn_mqa_fused_static_launch(const float *qkv, const int32_t *pos, const float *table, uint16_t *kc, uint16_t *vc,
                                  uint16_t *out, int hq, int dh, int max_ctx, hipStream_t st) {
     int dev = 0;
     CHADQ_HIP(hipGetDevice(&dev));
     CHADQ_REQUIRE(dev >= 0 && dev < 64, CHADQ_ERR_DEVICE, "attention without workspace: device index %d is not below 64", dev);
-    float *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
-    if (!ptr) {  // first call on this device (two threads racing here obtain the same address)
-        CHADQ_HIP(hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)));
-        CHADQ_REQUIRE(ptr != nullptr, CHADQ_ERR_HIP, "hipGetSymbolAddress returned a null address for the attention scratch");
-        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
-    }
+    float *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);  // set by the device's first entry-point call
+    CHADQ_REQUIRE(ptr != nullptr, CHADQ_ERR_HIP, "attention without workspace: the scratch address of device %d was not resolved", dev);
     if ((size_t)((max_ctx + ATT_CS - 1) / ATT_CS) * hq * (dh + 2) > ATT_STATIC_FLOATS)
         return fail(CHADQ_ERR_WORKSPACE, "attention without workspace: hq=%d dh=%d max_ctx=%d needs more than the %zu-float scratch", hq, dh,
                     max_ctx, ATT_STATIC_FLOATS);

@@ -14,8 +14,8 @@
 //              epilogue), each aligned run of 8 in the order 0,4,1,5,2,6,3,7 in which the dequantisation leaves the
 //              weights.  expert_prep_kernel writes them, gathered into expert order;
 //   correction sum_k x_k (u_k - 8) s_g = sum_k x_k u_k s_g - 8 s_g X_g with X_g the sum of the group's 32 activations:
-//              a second product with one term per scale group.  expert_prep_kernel also writes -8 X_g (fp16, as a high
-//              and a low part), and once per 512 k one pair of MFMAs per accumulator block multiplies them with the
+//              a second product with one term per scale group.  The preparation also writes -8 X_g (fp16, as a high and
+//              a low part), and once per 512 k one pair of MFMAs per accumulator block multiplies them with the
 //              lane's scales of those 512 k, which are exactly the 8 values it already holds in registers: 1/16 more
 //              matrix work instead of 4 more vector instructions per 8 weights.
 //

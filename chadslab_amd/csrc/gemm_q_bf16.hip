@@ -19,10 +19,13 @@
 // The MFMA k-slot of a lane is free to choose as long as A and B agree: slot group kq covers the kq-th
 // 16-byte weight load, and step t of that load is its t-th 8-k word.
 // The four partial tiles are summed through LDS at the end, rounded to bf16 (RNE) and stored coalesced.
-#include <cstdlib>
 #include <type_traits>
 
 #include "chadq_common.h"
+
+#ifndef CHADQ_GEMM_ABLATE
+#define CHADQ_GEMM_ABLATE 0  // measurement builds only: 1 = the dequantisation compiled out (packed words go to the matrix core as they are)
+#endif
 
 namespace chadq {
 
@@ -223,7 +226,10 @@ __global__ __launch_bounds__(256) void gemm_q_bf16_kernel(const uint16_t *__rest
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             const u32x4 q = cq[nb];
-            if constexpr (i4) {
+            if constexpr (CHADQ_GEMM_ABLATE == 1) {
+                const u32x4 raw = {q.x + (uint32_t)t, q.y, q.z, q.w};
+                __builtin_memcpy(&bf[set][t][nb], &raw, 16);
+            } else if constexpr (i4) {
                 const uint32_t wsel = t == 0 ? q.x : t == 1 ? q.y : t == 2 ? q.z : q.w;
                 bf[set][t][nb] = dequant8_i4(wsel, cs[nb][0], cs[nb][1], cs[nb][2], cs[nb][3], c_mlo, c_mhi, c_magic);
             } else {
@@ -430,14 +436,9 @@ int gemm_i4g32_bf16_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_
                              int K, hipStream_t st) {
     // many rows: the 256 x 256 tile, which dequantises a weight once per 256 rows, as soon as its tiles cover most of
     // the chip (a tile alone on a compute unit takes about as long as all of them together: at 4096 columns the small
-    // tile is still ahead at 2048 rows, 101 against 115 us).  CHADQ_GEMM_TILE=big / small overrides the choice.
-    static const int force = [] {
-        const char *e = getenv("CHADQ_GEMM_TILE");
-        return !e ? 0 : (e[0] == 'b' ? 1 : (e[0] == 's' ? -1 : 0));
-    }();
+    // tile is still ahead at 2048 rows, 101 against 115 us)
     const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-    if (force >= 0 && (force > 0 || big_tiles >= 176) && gemm_big_i4g32_ok(x, wp, sc, M, N, K))
-        return gemm_big_i4g32_launch(x, wp, sc, y, M, N, K, st);
+    if (big_tiles >= 176 && gemm_big_i4g32_ok(x, wp, sc, M, N, K)) return gemm_big_i4g32_launch(x, wp, sc, y, M, N, K, st);
     return launch_gemm<FmtI4G32, false>(x, wp, sc, y, M, N, K, nullptr, 0, st);
 }
 

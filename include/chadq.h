@@ -271,9 +271,11 @@ int chadq_attn_decode_mqa_fused(const float *qkv, const int32_t *pos, const floa
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments minus the
  * workspace, same kernels, same results bit for bit: the split-context partials live in a 2,113,536-byte array inside
  * the library's device code (one per GPU, held until the process ends), which covers max_ctx <= 8192 at hq <= 8,
- * dh <= 256; a larger max_ctx returns CHADQ_ERR_WORKSPACE.  Calls no hipMalloc / hipFree; the first call on a device
- * looks the array's address up (hipGetSymbolAddress), so make that call outside a stream capture.  Every call on a GPU
- * shares that GPU's array: calls that overlap on one GPU (different streams) race.
+ * dh <= 256; a larger max_ctx returns CHADQ_ERR_WORKSPACE.  Calls no hipMalloc / hipFree.  The array's address on a
+ * device is looked up (hipGetSymbolAddress) by the first call of ANY entry point of this library on that device, which
+ * therefore has to happen outside a stream capture (a repack, a warm-up step, chadq_rope_table all do); this entry
+ * point itself only reads the stored address.  Every call on a GPU shares that GPU's array: one call at a time per
+ * GPU - calls that overlap on one GPU (two streams, or two graphs replayed concurrently) race on it silently.
  */
 int chadq_attn_decode_mqa_fused_static(const float *qkv, const int32_t *pos, const float *rope_table, uint16_t *kcache_bf16,
                                        uint16_t *vcache_bf16, uint16_t *out_bf16, int hq, int dh, int max_ctx, void *stream);
