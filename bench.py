@@ -273,6 +273,27 @@ def main():
                         extras[name]["us_without_dequantisation"] = round(run_steps(lambda i: ops.qgemm(x2, qw, out=y2), *n_gemm)[0], 3)
                 finally:
                     _lib._lib = main_lib
+        # context: what the matrix cores sustain on non-zero operands with no memory traffic at all (bench_probe.hip)
+        import ctypes
+
+        probe_path = os.path.join(ROOT, "bench_probe.so")
+        if os.path.exists(probe_path):
+            plib2 = ctypes.CDLL(probe_path)
+            plib2.bench_probe_mfma.restype = ctypes.c_int
+            plib2.bench_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+            pbuf = torch.empty(512 * 256, dtype=torch.float32, device=dev)
+            trips = 400
+            sustained = {}
+            for kind, kname in ((0, "fp16"), (1, "bf16")):
+                def mf(i, kind=kind):
+                    if plib2.bench_probe_mfma(kind, trips, pbuf.data_ptr(), torch.cuda.current_stream().cuda_stream):
+                        raise RuntimeError("bench_probe_mfma failed")
+                usm = run_steps(mf, 24, 8)[0]
+                sustained[kname + "_TFLOPs"] = round(512 * 4 * trips * 24 * 32768.0 / usm * 1e-6, 1)
+            sustained["note"] = ("v_mfma_f32_32x32x16 on non-zero operands held in registers, 2 waves per SIMD, no memory traffic: the "
+                                 "matrix cores' practical ceiling on this machine (the clock follows the power drawn)")
+            extras["mfma_sustained_registers_only"] = sustained
+            del pbuf
         # context: the vendor library's plain bf16 GEMM (no dequantisation) on the same shape, through torch.matmul
         wb16 = torch.randn(N2, K2, device=dev).to(torch.bfloat16)
         yt = torch.empty(M2, N2, dtype=torch.bfloat16, device=dev)

@@ -47,3 +47,46 @@ extern "C" int bench_probe_empty(void *stream) {
     hipLaunchKernelGGL(probe_empty_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream);
     return (int)hipGetLastError();
 }
+
+// What the matrix cores sustain on operands that are not zero, registers only (no memory traffic at all): 512 workgroups
+// of four waves, six accumulator chains per wave, 4 x 6 MFMAs of 32 x 32 x 16 per trip.  The clock follows the power
+// the arithmetic draws, so this, not the nominal peak, is the ceiling of every matrix-core-bound kernel here.
+typedef __attribute__((ext_vector_type(8))) _Float16 probe_f16x8;
+typedef __attribute__((ext_vector_type(8))) __bf16 probe_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float probe_f32x16;
+
+template <int KIND>
+__global__ __launch_bounds__(256) void probe_mfma_kernel(float *__restrict__ out, int trips) {
+    probe_f32x16 acc[6];
+    for (int i = 0; i < 6; ++i)
+        for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+    probe_f16x8 a, b;
+    probe_bf16x8 ab, bb;
+    for (int e = 0; e < 8; ++e) {
+        a[e] = (_Float16)(0.37f * (float)((threadIdx.x * 7 + e) % 61) - 9.f);
+        b[e] = (_Float16)(0.11f * (float)((threadIdx.x * 3 + e + 1) % 53) - 2.f);
+        ab[e] = (__bf16)(float)a[e];
+        bb[e] = (__bf16)(float)b[e];
+    }
+    for (int t = 0; t < trips; ++t) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int i = 0; i < 6; ++i) {
+                if (KIND == 0) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i], 0, 0, 0);
+                else acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ab, bb, acc[i], 0, 0, 0);
+            }
+    }
+    float s = 0.f;
+    for (int i = 0; i < 6; ++i)
+        for (int v = 0; v < 16; ++v) s += acc[i][v];
+    out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+// kind 0: fp16, 1: bf16.  out: 512 * 256 floats.  flop per launch = 512 * 4 * trips * 24 * 32768.
+extern "C" int bench_probe_mfma(int kind, int trips, float *out, void *stream) {
+    if (!out || trips < 1 || kind < 0 || kind > 1) return -1;
+    if (kind == 0) hipLaunchKernelGGL(probe_mfma_kernel<0>, dim3(512), dim3(256), 0, (hipStream_t)stream, out, trips);
+    else hipLaunchKernelGGL(probe_mfma_kernel<1>, dim3(512), dim3(256), 0, (hipStream_t)stream, out, trips);
+    return (int)hipGetLastError();
+}
