@@ -52,6 +52,8 @@ SIGNATURES = {
     "chadq_attn_decode_mqa_fused_workspace_floats": (c_size_t, [c_int, c_int, c_int]),
     "chadq_attn_decode_mqa_fused": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                             c_void_p]),
+    "chadq_attn_decode_mqa_fused_oproj_i4g32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "chadq_attn_decode_mqa_fused_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                                    c_void_p]),
     "chadq_geglu_bf16": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),

@@ -83,6 +83,9 @@ int geglu_launch(const float *, uint16_t *, int, hipStream_t);
 int rope_table_launch(float *, int, int, float, hipStream_t);
 int attn_mqa_fused_launch(const float *, const int32_t *, const float *, uint16_t *, uint16_t *, float *, uint16_t *, int, int, int,
                           hipStream_t);
+bool attn_mqa_fused_oproj_ok(int hq, int dh);
+int attn_mqa_fused_oproj_launch(const float *, const int32_t *, const float *, uint16_t *, uint16_t *, float *, const uint8_t *,
+                                const uint16_t *, float *, int, int, int, int, hipStream_t);
 int attn_mqa_fused_static_launch(const float *, const int32_t *, const float *, uint16_t *, uint16_t *, uint16_t *, int, int, int,
                                  hipStream_t);
 int attn_mqa_fused_static_max_ctx();
@@ -404,6 +407,23 @@ int chadq_attn_decode_mqa_fused(const float *qkv, const int32_t *pos, const floa
     CHADQ_REQUIRE(aligned16(qkv) && aligned16(rope_table) && aligned16(kcache_bf16), CHADQ_ERR_ALIGN,
                   "chadq_attn_decode_mqa_fused: qkv, rope_table and kcache must be 16-byte aligned");
     return attn_mqa_fused_launch(qkv, pos, rope_table, kcache_bf16, vcache_bf16, workspace, out_bf16, hq, dh, max_ctx, st);
+}
+
+int chadq_attn_decode_mqa_fused_oproj_i4g32(const float *qkv, const int32_t *pos, const float *rope_table, uint16_t *kcache_bf16,
+                                            uint16_t *vcache_bf16, float *workspace, const uint8_t *wp,
+                                            const uint16_t *scale_f16, float *y_parts, int hq, int dh, int max_ctx, int N,
+                                            void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(attn_mqa_fused_oproj_ok(hq, dh) && max_ctx >= 1 && max_ctx <= 65536 && N >= 1, CHADQ_ERR_SHAPE,
+                  "chadq_attn_decode_mqa_fused_oproj_i4g32: hq=%d dh=%d max_ctx=%d N=%d (dh = 256, hq one of 2, 4, 6, 8, "
+                  "max_ctx <= 65536)", hq, dh, max_ctx, N);
+    CHADQ_REQUIRE(qkv && pos && rope_table && kcache_bf16 && vcache_bf16 && workspace && wp && scale_f16 && y_parts, CHADQ_ERR_NULL,
+                  "chadq_attn_decode_mqa_fused_oproj_i4g32: null pointer");
+    CHADQ_REQUIRE(aligned16(qkv) && aligned16(rope_table) && aligned16(kcache_bf16) && aligned16(workspace) && aligned16(wp),
+                  CHADQ_ERR_ALIGN,
+                  "chadq_attn_decode_mqa_fused_oproj_i4g32: qkv, rope_table, kcache, workspace and wp must be 16-byte aligned");
+    return attn_mqa_fused_oproj_launch(qkv, pos, rope_table, kcache_bf16, vcache_bf16, workspace, wp, scale_f16, y_parts, hq, dh,
+                                       max_ctx, N, st);
 }
 
 int chadq_attn_decode_mqa_fused_static(const float *qkv, const int32_t *pos, const float *rope_table, uint16_t *kcache_bf16,

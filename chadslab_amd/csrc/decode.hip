@@ -544,6 +544,143 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
     }
 }
 
+// ---- the combination of the partials folded into the output projection that consumes the attention vector ----
+// y_part[hp][n] = sum over the 512 k of head pair hp of Wo[n][k] * att[k], Wo int4 group-32 [N, hq*256], att the bf16 attention
+// vector attn_mqa_combine_kernel would have written.  A launch less per layer: the combination has no kernel of its own,
+// every workgroup of the projection forms the 512 attention values it multiplies with for itself.
+//
+// Workgroup (hp, row block): 16 waves, 64*NL weight rows.
+//   1. Wave w takes head 2*hp + (w & 1) and the slices b = (w >> 1) + 8i of each batch of 64: lane q fetches columns
+//      4q..4q+3 of those 8 slices (the rows of the workspace are 8-byte aligned only, hence the loads of that alignment)
+//      and lane b the running maximum and sum of slice b; every wave works out the factors exp(m_b - M) itself.  Batches
+//      beyond the first (contexts over 2048 positions) are folded in with the usual rescaling.  The workgroup's weight
+//      loads - one 16-byte load per lane and 4 rows: lane (r, g) holds scale group g of its row - are issued behind the
+//      first batch and land while the combination runs.
+//   2. The eight slice groups meet in LDS; thread c sums column c, divides, rounds to bf16 and stores it where the dot
+//      products want it: 16-byte pieces of 8 k in the pair order of unpack8_magic, piece t of group g at (16t + g) * 16
+//      (the 16 lanes of a row then read 256 consecutive bytes).
+//   3. dot products with v_dot2_f32_bf16 on 128+u, -136 * sum(x) per group, the lane's scale, a sum over the 16 lanes of
+//      the row.  The parts of the hq/2 head pairs are added by the consumer (the next projection's residual add).
+typedef float f32x4_a8 __attribute__((ext_vector_type(4), aligned(8)));
+
+template <int NL>
+__global__ __launch_bounds__(1024) void attn_combine_oproj_kernel(const float *__restrict__ part, const int32_t *__restrict__ pos,
+                                                                  const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
+                                                                  float *__restrict__ y, int hq, int max_ctx, int N) {
+    constexpr int dh = 256;
+    const int K = hq * dh, KH = K >> 1, G = K >> 5;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int hp = blockIdx.x, hl = wave & 1, sg = wave >> 1, h = 2 * hp + hl;
+    const int nbmax = (max_ctx + ATT_CS - 1) / ATT_CS;
+    __shared__ __attribute__((aligned(16))) float s_num[8][2 * dh];
+    __shared__ __attribute__((aligned(16))) uint8_t s_x[2 * dh * 2];
+    __shared__ float s_den[2];
+
+    const int pos0 = pos[0];  // asked for first: the only load the factors of the first batch wait for besides their own
+    const size_t stride = (size_t)hq * (dh + 2);
+    const float *ph = part + (size_t)h * (dh + 2);
+    const int bl = lane < nbmax ? lane : nbmax - 1;
+    const float m0 = ph[(size_t)bl * stride], l0 = ph[(size_t)bl * stride + 1];
+    f32x4 pre[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int b = sg + 8 * i;
+        pre[i] = *reinterpret_cast<const f32x4_a8 *>(ph + (size_t)(b < nbmax ? b : nbmax - 1) * stride + 2 + 4 * lane);
+    }
+    const int r = lane >> 4, g = lane & 15;
+    const int n0 = (blockIdx.y * 16 + wave) * 4 * NL;
+    u32x4 w[NL];
+    uint16_t sw[NL];
+#pragma unroll
+    for (int l = 0; l < NL; ++l) {
+        const int row = n0 + 4 * l + r, rowc = row < N ? row : N - 1;
+        w[l] = load_nt_b128(wp + (size_t)rowc * KH + (size_t)(hp * 16 + g) * 16);
+        sw[l] = sc[(size_t)rowc * G + hp * 16 + g];
+    }
+    const int ctx = min(max(pos0, 0), max_ctx - 1) + 1, nb = (ctx + ATT_CS - 1) / ATT_CS;
+    __builtin_amdgcn_sched_barrier(0);
+
+    float M = wave_max_all(lane < nb ? m0 : -INFINITY);
+    const float f0 = lane < nb ? __expf(m0 - M) : 0.f;
+    float den = lane < nb ? f0 * l0 : 0.f;
+    f32x4 num = {0.f, 0.f, 0.f, 0.f};
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        // a slice past the context holds whatever the workspace held: selected away, not multiplied by zero (and not
+        // skipped by a branch, which would move its load behind the branch)
+        const int b = sg + 8 * i;
+        num += lane_value(f0, b) * (b < nb ? pre[i] : zero4);
+    }
+    for (int base = 64; base < nb; base += 64) {
+        const int b = base + lane;
+        const bool in = b < nb;
+        const float mb = in ? ph[(size_t)b * stride] : -INFINITY, lb = in ? ph[(size_t)b * stride + 1] : 0.f;
+        f32x4 pv[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int bb = base + sg + 8 * i;  // uniform over the wave
+            pv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (bb < nb) pv[i] = *reinterpret_cast<const f32x4_a8 *>(ph + (size_t)bb * stride + 2 + 4 * lane);
+        }
+        const float Mn = fmaxf(M, wave_max_all(mb));
+        const float rs = __expf(M - Mn), f = in ? __expf(mb - Mn) : 0.f;
+        den = den * rs + f * lb;
+        num *= rs;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (base + sg + 8 * i < nb) num += lane_value(f, sg + 8 * i) * pv[i];
+        M = Mn;
+    }
+    den = wave_sum_to_lane63(den);
+    *reinterpret_cast<f32x4 *>(&s_num[sg][hl * dh + 4 * lane]) = num;
+    if (sg == 0 && lane == 63) s_den[hl] = den;
+    __syncthreads();
+    if (tid < 2 * dh) {
+        float t = s_num[0][tid];
+#pragma unroll
+        for (int s8 = 1; s8 < 8; ++s8) t += s_num[s8][tid];
+        const int gg = tid >> 5, tt = (tid >> 3) & 3, e = tid & 7;
+        *reinterpret_cast<uint16_t *>(s_x + (tt * 16 + gg) * 16 + (e & 3) * 4 + (e >> 2) * 2) =
+            (uint16_t)f32_to_bf16_bits(t / s_den[tid >> 8]);
+    }
+    __syncthreads();
+
+    u32x4 xv[4];
+    float sumx = 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        xv[t] = *reinterpret_cast<const u32x4 *>(s_x + (t * 16 + g) * 16);
+        sumx = dot2_bf16(xv[t].x, 0x3F803F80u, sumx);
+        sumx = dot2_bf16(xv[t].y, 0x3F803F80u, sumx);
+        sumx = dot2_bf16(xv[t].z, 0x3F803F80u, sumx);
+        sumx = dot2_bf16(xv[t].w, 0x3F803F80u, sumx);
+    }
+    const uint32_t mask_r = vgpr_const(0x000F000Fu), magic_r = vgpr_const(kBf16Magic);
+#pragma unroll
+    for (int l = 0; l < NL; ++l) {
+        const uint32_t ww[4] = {w[l].x, w[l].y, w[l].z, w[l].w};
+        float acc = 0.f;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            uint32_t pw[4];
+            unpack8_magic_r(ww[t], mask_r, magic_r, pw);
+            acc = dot2_bf16(pw[0], xv[t].x, acc);
+            acc = dot2_bf16(pw[1], xv[t].y, acc);
+            acc = dot2_bf16(pw[2], xv[t].z, acc);
+            acc = dot2_bf16(pw[3], xv[t].w, acc);
+        }
+        float v = f16_bits_to_f32(sw[l]) * (acc - kMagicBias * sumx);
+        v += dpp_f32<0x128, 0xF>(v);  // row_ror:8
+        v += dpp_f32<0x124, 0xF>(v);  // row_ror:4
+        v += dpp_f32<0x122, 0xF>(v);  // row_ror:2
+        v += dpp_f32<0x121, 0xF>(v);  // row_ror:1: every lane of the 16-lane row holds the row's sum
+        const int row = n0 + 4 * l + r;
+        if (g == 0 && row < N) y[(size_t)hp * N + row] = v;
+    }
+}
+
 // h = bf16( gelu_tanh(g) * u ), gu = [g(F) | u(F)] fp32
 __global__ __launch_bounds__(256) void geglu_kernel(const float *__restrict__ gu, uint16_t *__restrict__ h, int F) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -682,6 +819,23 @@ int attn_mqa_fused_launch(const float *qkv, const int32_t *pos, const float *tab
     hipLaunchKernelGGL(attn_mqa_fused_kernel, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, out, hq, dh, max_ctx);
     hipLaunchKernelGGL(attn_mqa_combine_kernel, dim3(hq, (dh + 63) / 64), dim3(256), 0, st, ws, pos, out, hq, dh, max_ctx);
     return hip_check(hipGetLastError(), "attn_mqa_fused launch");
+}
+
+// The fused attention with its combination folded into the output projection: two launches for what were three
+// (partials, combination, projection).  y receives hq/2 partial vectors of N floats.
+bool attn_mqa_fused_oproj_ok(int hq, int dh) { return dh == 256 && hq >= 2 && hq <= 8 && hq % 2 == 0; }
+
+int attn_mqa_fused_oproj_launch(const float *qkv, const int32_t *pos, const float *table, uint16_t *kc, uint16_t *vc, float *ws,
+                                const uint8_t *wp, const uint16_t *sc, float *y, int hq, int dh, int max_ctx, int N, hipStream_t st) {
+    const int nb = (max_ctx + ATT_CS - 1) / ATT_CS;
+    hipLaunchKernelGGL(attn_mqa_fused_kernel, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, (uint16_t *)nullptr, hq, dh,
+                       max_ctx);
+    // 64 rows per workgroup up to 4096 rows (hq/2 * N/64 workgroups: 128 for a 2048-row matrix), 128 beyond
+    if (N <= 4096)
+        hipLaunchKernelGGL((attn_combine_oproj_kernel<1>), dim3(hq / 2, (N + 63) / 64), dim3(1024), 0, st, ws, pos, wp, sc, y, hq, max_ctx, N);
+    else
+        hipLaunchKernelGGL((attn_combine_oproj_kernel<2>), dim3(hq / 2, (N + 127) / 128), dim3(1024), 0, st, ws, pos, wp, sc, y, hq, max_ctx, N);
+    return hip_check(hipGetLastError(), "attn_mqa_fused_oproj launch");
 }
 
 // ---- the fused attention without a caller-supplied workspace ---------------------------------------------------

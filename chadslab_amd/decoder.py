@@ -96,7 +96,11 @@ class QuantDecoder:
         self.x, self.x2, self.xn = z(c.d, f32), z(c.d, f32), z(c.d, bf16)  # the residual stream ping-pongs between x and x2
         self.fused_norm1 = c.d % 256 == 0 and c.d <= 2048  # first norm of a layer folded into the qkv projection
         self.qkv, self.q = z((c.hq + 2) * c.dh, f32), z(c.hq * c.dh, f32)
-        self.att, self.ao = z(c.hq * c.dh, bf16), z(c.d, f32)
+        # the combination of the attention partials folded into the o projection, which then leaves one partial vector
+        # per pair of heads for the next residual add (the entry point's rules: dh = 256, an even hq; the adds that
+        # follow take up to four vectors)
+        self.fused_oproj = c.dh == 256 and c.hq in (2, 4, 6, 8) and c.max_ctx <= 65536
+        self.att, self.ao = z(c.hq * c.dh, bf16), z((c.hq // 2 if self.fused_oproj else 1) * c.d, f32)
         # the down projection has few rows and a long K: split it over K when that fills the chip better
         self.ksplit = next((s for s in (4, 2) if c.ffn % (s * 4096) == 0), 1)
         self.gu, self.h, self.dn = z(2 * c.ffn, f32), z(c.ffn, bf16), z(self.ksplit * c.d, f32)
@@ -168,7 +172,12 @@ class QuantDecoder:
                 self._gemv(self.xn, L["wqkv"], self.qkv)
             if trace is not None:
                 trace.append(self.x.clone())  # the pending down projection has just been added: the layer's input
-            if self.fused_attn:
+            if self.fused_attn and self.fused_oproj:
+                _lib.check(lib.chadq_attn_decode_mqa_fused_oproj_i4g32(
+                    self.qkv.data_ptr(), self.pos.data_ptr(), self.rope.data_ptr(), self.kcache[li].data_ptr(),
+                    self.vcache[li].data_ptr(), self.part.data_ptr(), L["wo"].packed.data_ptr(), L["wo"].scale.data_ptr(),
+                    self.ao.data_ptr(), c.hq, c.dh, c.max_ctx, c.d, s), "chadq_attn_decode_mqa_fused_oproj_i4g32")
+            elif self.fused_attn:
                 _lib.check(lib.chadq_attn_decode_mqa_fused(self.qkv.data_ptr(), self.pos.data_ptr(), self.rope.data_ptr(),
                                                            self.kcache[li].data_ptr(), self.vcache[li].data_ptr(),
                                                            self.part.data_ptr(), self.att.data_ptr(), c.hq, c.dh, c.max_ctx, s),
@@ -180,10 +189,12 @@ class QuantDecoder:
                 _lib.check(lib.chadq_attn_decode_mqa(self.q.data_ptr(), self.kcache[li].data_ptr(), self.vcache[li].data_ptr(),
                                                      self.pos.data_ptr(), self.part.data_ptr(), self.att.data_ptr(), c.hq, c.dh,
                                                      c.max_ctx, s), "chadq_attn_decode_mqa")
-            self._gemv(self.att, L["wo"], self.ao)
+            if not (self.fused_attn and self.fused_oproj):
+                self._gemv(self.att, L["wo"], self.ao)
+            nao = self.ao.numel() // c.d
             if self.fused_geglu:  # the second norm folds into the gate+up projection, the GeGLU into its epilogue
                 wil = self.wgu_il[li]
-                _lib.check(lib.chadq_gemv_i4g32_addnorm_geglu(self.x.data_ptr(), self.ao.data_ptr(), 1, L["ln2"].data_ptr(), c.eps,
+                _lib.check(lib.chadq_gemv_i4g32_addnorm_geglu(self.x.data_ptr(), self.ao.data_ptr(), nao, L["ln2"].data_ptr(), c.eps,
                                                               self.x2.data_ptr(), wil.packed.data_ptr(), wil.scale.data_ptr(),
                                                               self.h.data_ptr(), wil.N, c.d, s), "chadq_gemv_i4g32_addnorm_geglu")
                 self.x, self.x2 = self.x2, self.x

@@ -267,6 +267,22 @@ int chadq_attn_decode_mqa_fused(const float *qkv, const int32_t *pos, const floa
                                 void *stream);
 
 /*
+ * chadq_attn_decode_mqa_fused followed by the output projection that consumes its result, y = Wo * out with Wo an int4
+ * group-32 matrix [N, hq*dh] (wp / scale_f16 as for chadq_gemv_i4g32), in two launches instead of three: the
+ * combination of the split-context partials happens inside the projection.  The projection is split over K by pairs
+ * of heads: y_parts fp32 [hq/2, N] receives one partial vector per pair and the caller (or the n_delta argument of
+ * chadq_gemv_i4g32_addnorm / _addnorm_geglu / chadq_add_rmsnorm_bf16) adds them, in order.  The attention vector itself
+ * is rounded to bf16 as chadq_attn_decode_mqa_fused rounds it, but is not written anywhere.
+ * dh = 256 and hq in {2, 4, 6, 8} (CHADQ_ERR_SHAPE otherwise: use the two separate calls), max_ctx <= 65536, N >= 1;
+ * qkv, rope_table, kcache, workspace and wp 16-byte aligned.  Workspace as chadq_attn_decode_mqa_fused_workspace_floats.
+ * The reference has no counterpart: its numpy runtime would call the attention and the projection one after the other.
+ */
+int chadq_attn_decode_mqa_fused_oproj_i4g32(const float *qkv, const int32_t *pos, const float *rope_table, uint16_t *kcache_bf16,
+                                            uint16_t *vcache_bf16, float *workspace, const uint8_t *wp,
+                                            const uint16_t *scale_f16, float *y_parts, int hq, int dh, int max_ctx, int N,
+                                            void *stream);
+
+/*
  * chadq_attn_decode_mqa_fused for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments minus the
  * workspace, same kernels, same results bit for bit: the split-context partials live in a 2,113,536-byte array inside

@@ -283,6 +283,72 @@ def test_attn_decode_mqa_fused_equals_rope_write_attend(lib, hq, dh, pos, max_ct
     assert np.array_equal(kb[rest], kc[rest])
 
 
+@pytest.mark.parametrize("hq,pos,max_ctx,n", [(8, 0, 64, 2048), (8, 31, 64, 2048), (8, 32, 4096, 2048), (8, 2047, 4096, 2048),
+                                              (8, 2048, 4096, 2048), (8, 2111, 4096, 2048), (8, 4095, 4096, 2048),
+                                              (8, 8191, 8192, 2048), (2, 70, 128, 100), (4, 300, 512, 4100), (6, 129, 256, 65)])
+def test_attn_fused_oproj_equals_attention_then_projection(lib, hq, pos, max_ctx, n):
+    """The output projection with the combination of the attention partials folded in, against (a) the separate calls on the
+    GPU - the same bf16 attention vector through the oracle's f64 GEMV, and identical caches - and (b) the oracle end to end."""
+    dh, k = 256, hq * 256
+    r = rng(11 * hq + pos + n)
+    qkv = r.standard_normal((hq + 2) * dh).astype(np.float32)
+    kc = O.f32_to_bf16(r.standard_normal((max_ctx, dh)).astype(np.float32))
+    vc = O.f32_to_bf16(r.standard_normal((max_ctx, dh)).astype(np.float32))
+    u = r.integers(0, 16, (n, k), dtype=np.uint8)
+    packed = (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8)
+    sc = r.lognormal(-5, 0.5, (n, k // 32)).astype(np.float16)
+    tq, tp = dev(qkv), torch.tensor([pos], dtype=torch.int32, device=DEV)
+    tw, ts = dev(packed), dev(sc)
+    table = torch.zeros(max_ctx * dh, dtype=torch.float32, device=DEV)
+    chk(lib.chadq_rope_table(table.data_ptr(), dh, max_ctx, 10000.0, stream()), "table")
+    nws = lib.chadq_attn_decode_mqa_fused_workspace_floats(hq, dh, max_ctx)
+    # separate calls
+    tk1, tv1 = bf16_tensor(kc.reshape(-1)), bf16_tensor(vc.reshape(-1))
+    ws1 = torch.zeros(nws, dtype=torch.float32, device=DEV)
+    att = torch.zeros(k, dtype=torch.bfloat16, device=DEV)
+    chk(lib.chadq_attn_decode_mqa_fused(tq.data_ptr(), tp.data_ptr(), table.data_ptr(), tk1.data_ptr(), tv1.data_ptr(),
+                                        ws1.data_ptr(), att.data_ptr(), hq, dh, max_ctx, stream()), "attn fused")
+    # one call; the workspace starts out full of NaN: slices past the context must never reach a sum
+    tk2, tv2 = bf16_tensor(kc.reshape(-1)), bf16_tensor(vc.reshape(-1))
+    ws2 = torch.full((nws,), float("nan"), dtype=torch.float32, device=DEV)
+    parts = torch.full((hq // 2, n), float("nan"), dtype=torch.float32, device=DEV)
+    for call in range(2):  # the second call finds the new row already in the cache
+        chk(lib.chadq_attn_decode_mqa_fused_oproj_i4g32(tq.data_ptr(), tp.data_ptr(), table.data_ptr(), tk2.data_ptr(),
+                                                        tv2.data_ptr(), ws2.data_ptr(), tw.data_ptr(), ts.data_ptr(),
+                                                        parts.data_ptr(), hq, dh, max_ctx, n, stream()), "attn fused oproj")
+        torch.cuda.synchronize()
+        got = parts.cpu().numpy()
+        assert np.isfinite(got).all(), "call %d" % call
+        assert np.array_equal(bits(tk2), bits(tk1)) and np.array_equal(bits(tv2), bits(tv1))
+        # (a) per pair of heads, on the attention vector the separate kernel rounded to bf16: the two combinations may
+        # round a value to neighbouring bf16 numbers, nothing more
+        ab = bits(att)
+        for hp in range(hq // 2):
+            xb = np.zeros((1, k), dtype=np.uint16)
+            xb[0, hp * 512:(hp + 1) * 512] = ab[hp * 512:(hp + 1) * 512]
+            assert O.rel_l2(got[hp], O.qgemm_int4g32_f64(xb, packed, sc)[0]) < 3e-3, "call %d pair %d" % (call, hp)
+    # (b) the oracle: rotate, write the cache row, attend, round, project
+    q = O.rope_rotate_half(qkv[: hq * dh].reshape(hq, dh), pos)
+    kc[pos] = O.f32_to_bf16(O.rope_rotate_half(qkv[hq * dh: (hq + 1) * dh], pos))
+    vc[pos] = O.f32_to_bf16(qkv[(hq + 1) * dh:])
+    kk = O.bf16_to_f32(kc[: pos + 1]).astype(np.float64)
+    vv = O.bf16_to_f32(vc[: pos + 1]).astype(np.float64)
+    sco = q.astype(np.float64) @ kk.T / np.sqrt(dh)
+    pr = np.exp(sco - sco.max(-1, keepdims=True))
+    want_att = ((pr / pr.sum(-1, keepdims=True)) @ vv).astype(np.float32).reshape(1, k)
+    want = O.qgemm_int4g32_f64(O.f32_to_bf16(want_att), packed, sc)[0]
+    assert O.rel_l2(got.sum(0), want) < 1e-2
+
+
+def test_attn_fused_oproj_refuses_shapes_it_does_not_cover(lib):
+    z = torch.zeros(4096, dtype=torch.float32, device=DEV)
+    for hq, dh in ((3, 256), (8, 128), (10, 256), (0, 256)):
+        with pytest.raises(ValueError):
+            chk(lib.chadq_attn_decode_mqa_fused_oproj_i4g32(z.data_ptr(), z.data_ptr(), z.data_ptr(), z.data_ptr(), z.data_ptr(),
+                                                            z.data_ptr(), z.data_ptr(), z.data_ptr(), z.data_ptr(), hq, dh, 64,
+                                                            16, stream()), "attn fused oproj")
+
+
 def test_rope_table_matches_the_rotation(lib):
     dh, ctx = 64, 300
     table = torch.zeros(ctx * dh, dtype=torch.float32, device=DEV)
