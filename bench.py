@@ -63,6 +63,8 @@ def parse():
                          "adds, to gemm, config 2 on the build without dequantisation)")
     ap.add_argument("--short", action="store_true",
                     help="few launches per side measurement: for hardware-counter runs, which serialise every dispatch")
+    ap.add_argument("--settle-ms", type=float, default=40.0,
+                    help="run each measured workload for this long, untimed, right before its warm-up steps (0: not at all)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run three 256 MiB device copies before the timed region: a kernel of known traffic "
                          "that hardware-counter runs scale FETCH_SIZE / WRITE_SIZE by")
@@ -92,11 +94,60 @@ def main():
     def bits(t):
         return t.view(torch.int16).cpu().numpy().view(np.uint16)
 
-    def run_steps(fn, steps, warmup):
+    COVER = 24  # untimed launches queued in front of the start event (see run_direct)
+
+    def settle(fn, per_call=1):
+        """Runs the workload about to be measured for --settle-ms without a pause, untimed, in front of its warm-up
+        steps.  A GPU coming out of idle goes through a transient of some ten milliseconds (fast at first, then slower
+        than it will be, then steady), and the W warm-up steps of a 7 us kernel end inside it; the figures reported
+        are those of the steady state a decode loop runs in.  The headline's figure without this phase is reported
+        beside it.  fn(i) is called until the time is up; per_call = steps per call (a replayed graph)."""
+        if args.settle_ms <= 0:
+            return
+        t_end = time.perf_counter() + args.settle_ms * 1e-3
+        i = 0
+        while time.perf_counter() < t_end:
+            for _ in range(32):
+                fn(i)
+                i += per_call
+            if i % (32 * 64 * per_call) == 0:
+                torch.cuda.synchronize()  # bounds the backlog: the host may be faster than the GPU
+
+    def run_direct(fn, steps, warmup, do_settle=True):
+        """The steps as plain launches on the stream, one call of fn per step, back to back: `warmup` untimed steps, a
+        synchronize, then COVER more untimed steps that are already queued when the start event is recorded - the timed
+        steps are submitted while the GPU is still busy, so the cost of getting a first launch to an idle GPU is not
+        spread over them, however few they are - then exactly `steps` timed steps between two events on the launch stream.
+        Valid only while the host stays ahead of the GPU: returns None when its time per launch is not well below the
+        GPU's time per step (the caller then measures the same steps replayed from a captured graph)."""
+        with torch.cuda.stream(stream):
+            if do_settle:
+                settle(fn)
+            for i in range(max(1, warmup)):
+                fn(i)
+            torch.cuda.synchronize()
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            for i in range(COVER):
+                fn(i)
+            a.record(stream)
+            t0 = time.perf_counter()
+            for i in range(steps):
+                fn(COVER + i)
+            t1 = time.perf_counter()
+            b.record(stream)
+            torch.cuda.synchronize()
+        us, host = a.elapsed_time(b) * 1000.0 / steps, (t1 - t0) * 1e6 / steps
+        return (us, host, 0) if host < 0.75 * us else None
+
+    def run_steps(fn, steps, warmup, direct=False, do_settle=True):
         """fn(i) launches step i on the current stream.  Returns (us per step from HIP events, wall us per step,
-        launches per replayed graph).  The start event is recorded behind one more untimed replay that is already
-        queued, so the timed replays are submitted while the GPU is still busy: the cost of getting a graph launch
-        to an idle GPU is then not spread over the timed steps, however few they are."""
+        launches per replayed graph - 0 for plain stream launches).  direct: try run_direct first.  Graph form: the start
+        event is recorded behind one more untimed replay that is already queued, for the reason given in run_direct."""
+        if direct:
+            res = run_direct(fn, steps, warmup, do_settle)
+            if res is not None:
+                return res
         seg = min(SEG, steps)
         with torch.cuda.stream(stream):
             graphs = {}
@@ -110,6 +161,8 @@ def main():
                         fn(i)
                 graphs[length] = g
             full, rem = divmod(steps, seg)
+            if do_settle:
+                settle(lambda i: graphs[seg].replay(), seg)
             for _ in range(max(1, warmup // seg)):
                 graphs[seg].replay()
             torch.cuda.synchronize()
@@ -149,7 +202,26 @@ def main():
     def gemv_bytes(m):
         return N * K // 2 + N * (K // 32) * 2 + m * K * 2 + m * N * 4
 
+    def bound_step(fn, argv):
+        """step(i) = fn(*argv[i % len(argv)]), return codes OR-ed into step.rc."""
+        n = len(argv)
+
+        def step(i):
+            step.rc |= fn(*argv[i % n])
+
+        step.rc = 0
+        return step
+
+    def gemv_step(x, weights, y, m):
+        """step(i): one call of chadq_gemv_i4g32 on weight copy i % len(weights), arguments bound beforehand (a ctypes call
+        costs the host about 3 us, well under the kernel's time).  Return codes are OR-ed into step.rc."""
+        return bound_step(_lib.load().chadq_gemv_i4g32,
+                          [(x.data_ptr(), w.packed.data_ptr(), w.scale.data_ptr(), y.data_ptr(), m, N, K, stream.cuda_stream)
+                           for w in weights])
+
     want = set() if args.no_extras else {e for e in args.extras.split(",") if e}
+    if args.short:
+        args.settle_ms = 0.0  # hardware-counter runs serialise every dispatch: no phase that only spends launches
     n_side = (48, 24) if args.short else (480, 48)   # launches, warm-up of the GEMV side measurements
     n_gemm = (24, 24) if args.short else (240, 24)
     n_moe = 3 if args.short else 20
@@ -157,31 +229,32 @@ def main():
     results = {}
     parity = {}
     host = {}  # host copies of the side measurements' inputs, for the CPU legs
-    for m in (1, 4, 8):
-        if m != 1 and "gemv" not in want:
-            continue
-        x = torch.from_numpy(x_np[m]).to(torch.bfloat16).to(dev)
-        y = torch.empty(m, N, dtype=torch.float32, device=dev)
-        steps = args.steps if m == 1 else min(args.steps, n_side[0])
-        us, wall, seg_used = run_steps(lambda i: ops.qgemv(x, copies[i % N_COPIES], out=y), steps, args.warmup)
-        results[m] = (us, wall, steps, seg_used)
-        if m == 1:
-            from oracle import chadq_oracle as O  # the checker, used once outside the timed region
+    xs = {m: torch.from_numpy(x_np[m]).to(torch.bfloat16).to(dev) for m in (1, 4, 8)}
+    ys = {m: torch.empty(m, N, dtype=torch.float32, device=dev) for m in (1, 4, 8)}
 
-            parity["gemv_i4g32_m1_rel_l2_vs_f64"] = O.rel_l2(y.cpu().numpy(), O.qgemm_int4g32_f64(bits(x), packed, scale))
-    us1, wall1, steps1, seg1 = results[1]
-    achieved = gemv_bytes(1) / us1 * 1e-3  # GB/s
+    def measure_gemv(m, do_settle=True):
+        steps = args.steps if m == 1 else min(args.steps, n_side[0])
+        ops.qgemv(xs[m], copies[0], out=ys[m])  # once through the checked wrapper; the timed steps call the entry point itself
+        step = gemv_step(xs[m], copies, ys[m], m)
+        us, wall, seg_used = run_steps(step, steps, args.warmup, direct=True, do_settle=do_settle)
+        if step.rc:
+            raise RuntimeError("chadq_gemv_i4g32 returned %d during the timed steps" % step.rc)
+        return us, wall, steps, seg_used
+
+    # The headline measurement is taken twice: as the first thing this process runs on the GPU, with nothing but the W
+    # warm-up steps in front of it, and again at the end of the GEMV measurements behind a settling phase (settle()
+    # above).  The second figure is the one reported; the first is kept beside it in extras.
+    first_m1 = measure_gemv(1, do_settle=False)
+    from oracle import chadq_oracle as O  # the checker, used once outside the timed region
+
+    parity["gemv_i4g32_m1_rel_l2_vs_f64"] = O.rel_l2(ys[1].cpu().numpy(), O.qgemm_int4g32_f64(bits(xs[1]), packed, scale))
 
     extras = {}
     if "gemv" in want:
         x1 = torch.from_numpy(x_np[1]).to(torch.bfloat16).to(dev)
         y1 = torch.empty(1, N, dtype=torch.float32, device=dev)
-        us_hot = run_steps(lambda i: ops.qgemv(x1, base, out=y1), *n_side)[0]
-        extras["gemv_i4g32"] = {
-            "M%d" % m: {"us": round(results[m][0], 3), "GBps": round(gemv_bytes(m) / results[m][0] * 1e-3, 1),
-                        "frac_hbm_peak": round(gemv_bytes(m) / results[m][0] * 1e-3 / HBM_PEAK_GBS, 4)}
-            for m in results
-        }
+        us_hot = run_steps(gemv_step(x1, [base], y1, 1), *n_side, direct=True)[0]
+        extras["gemv_i4g32"] = {}
         extras["gemv_i4g32"]["M1_same_buffer_every_step"] = {
             "us": round(us_hot, 3), "GBps": round(gemv_bytes(1) / us_hot * 1e-3, 1),
             "note": "weights served by the 256 MB last-level cache, not HBM; not a roofline figure"}
@@ -198,11 +271,13 @@ def main():
             flat = [torch.empty(nread, dtype=torch.uint8, device=dev).fill_(i + 1) for i in range(N_COPIES)]
             pout = torch.empty(nread // 16384, dtype=torch.int32, device=dev)
 
+            pargs = [(f.data_ptr(), nread, pout.data_ptr(), stream.cuda_stream) for f in flat]
+
             def probe(i):
-                if plib.bench_probe_read(flat[i % N_COPIES].data_ptr(), nread, pout.data_ptr(), torch.cuda.current_stream().cuda_stream):
+                if plib.bench_probe_read(*pargs[i % N_COPIES]):
                     raise RuntimeError("bench_probe_read failed")
 
-            us_rd = run_steps(probe, *n_side)[0]
+            us_rd = run_steps(probe, *n_side, direct=True)[0]
             extras["gemv_i4g32"]["cold_read_same_bytes"] = {
                 "us": round(us_rd, 3), "GBps": round(nread / us_rd * 1e-3, 1), "bytes": int(nread),
                 "note": "loads only (bench_probe.hip), rotating buffers: the machine's ceiling for a read of this size"}
@@ -217,6 +292,19 @@ def main():
 
             extras["launch_floor_us"] = {"us": round(run_steps(empty, *n_side)[0], 3),
                                          "note": "an empty kernel (bench_probe.hip) per step, dependent launches in a replayed graph"}
+    if "gemv" in want:
+        for m in (4, 8):
+            results[m] = measure_gemv(m)
+    results[1] = measure_gemv(1)  # the reported one (see above)
+    us1, wall1, steps1, seg1 = results[1]
+    achieved = gemv_bytes(1) / us1 * 1e-3  # GB/s
+    if "gemv" in want:
+        for m in (1, 4, 8):
+            extras["gemv_i4g32"]["M%d" % m] = {"us": round(results[m][0], 3), "GBps": round(gemv_bytes(m) / results[m][0] * 1e-3, 1),
+                                               "frac_hbm_peak": round(gemv_bytes(m) / results[m][0] * 1e-3 / HBM_PEAK_GBS, 4)}
+    extras["gemv_i4g32_M1_first_measurement_of_the_process"] = {
+        "us": round(first_m1[0], 3), "GBps": round(gemv_bytes(1) / first_m1[0] * 1e-3, 1),
+        "note": "the same %d steps after %d warm-up steps and no settling phase, on a GPU that was idle until then" % (first_m1[2], args.warmup)}
     del copies
 
     if "int8" in want:
@@ -228,7 +316,16 @@ def main():
         x0, w0, s0 = (torch.from_numpy(a).to(dev) for a in host["cfg0"])
         c0 = [QWeightInt8(w0.clone(), s0.clone()) for _ in range(N_COPIES)]
         y0 = torch.empty(1, N0, dtype=torch.float32, device=dev)
-        us0 = run_steps(lambda i: ops.qgemv(x0, c0[i % N_COPIES], out=y0), *n_side)[0]
+        ops.qgemv(x0, c0[0], out=y0)  # once through the checked wrapper
+
+        def i8_step(xx, yy, m):
+            return bound_step(_lib.load().chadq_gemv_i8row, [(xx.data_ptr(), c.w.data_ptr(), c.scale.data_ptr(), yy.data_ptr(), m, N0, K0,
+                                                              stream.cuda_stream) for c in c0])
+
+        st0 = i8_step(x0, y0, 1)
+        us0 = run_steps(st0, *n_side, direct=True)[0]
+        if st0.rc:
+            raise RuntimeError("chadq_gemv_i8row returned %d during the timed steps" % st0.rc)
         b0 = N0 * K0 + N0 * 4 + K0 * 4 + N0 * 4
         extras["gemv_i8row_config0"] = {"us": round(us0, 3), "GBps": round(b0 / us0 * 1e-3, 1),
                                         "frac_hbm_peak": round(b0 / us0 * 1e-3 / HBM_PEAK_GBS, 4)}
@@ -236,7 +333,7 @@ def main():
         for m in (8, 16):
             xm = torch.from_numpy(r0.standard_normal((m, K0)).astype(np.float32)).to(dev)
             ym = torch.empty(m, N0, dtype=torch.float32, device=dev)
-            usm = run_steps(lambda i: ops.qgemv(xm, c0[i % N_COPIES], out=ym), *n_side)[0]
+            usm = run_steps(i8_step(xm, ym, m), *n_side, direct=True)[0]
             bm = N0 * K0 + N0 * 4 + m * (K0 * 4 + N0 * 4)
             extras["gemv_i8row_config0"][f"M{m}_extra"] = {"us": round(usm, 3), "GBps": round(bm / usm * 1e-3, 1)}
         del c0, w0
@@ -343,6 +440,7 @@ def main():
 
         def time_moe(ex):
             with torch.cuda.stream(stream):
+                settle(lambda i: ops.moe_ffn(x3, z3, ex))
                 for _ in range(3):
                     ops.moe_ffn(x3, z3, ex)
                 a3, b3 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -409,6 +507,8 @@ def main():
             dec.token.fill_(5)
             dec.pos.fill_(2040)
             dec.capture()
+            settle(lambda i: dec.graph.replay())  # positions 2040 .. about 2105 (max_ctx 4096); then back to the start
+            dec.pos.fill_(2040)
             for _ in range(8):
                 dec.graph.replay()
             a4, b4 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -437,6 +537,8 @@ def main():
             dec.pos.fill_(2040)
             dec.set_sampling(50, 1.0, 1004)
             dec.capture()
+            settle(lambda i: dec.graph.replay())
+            dec.pos.fill_(2040)
             for _ in range(8):
                 dec.graph.replay()
             a4, b4 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -592,13 +694,18 @@ def main():
         "dtype": "bf16 x int4 -> fp32 accumulate",
         "data": "synthetic",
         "config": {"workload": "config 1: int4 group-32 decode GEMV, M=1, W [14336,4096], x bf16, y fp32",
-                   "M": 1, "N": N, "K": K, "weight_copies_rotated": N_COPIES, "launch": "HIP graph replay, %d launches per graph" % seg1,
-                   "algorithmic_bytes_per_launch": gemv_bytes(1)},
+                   "M": 1, "N": N, "K": K, "weight_copies_rotated": N_COPIES, "launch": ("HIP graph replay, %d launches per graph" % seg1) if seg1 else
+                   ("one chadq_gemv_i4g32 call per step on one stream, back to back (host %.1f us per call); %d untimed steps "
+                    "queued in front of the start event" % (wall1, COVER)),
+                   "algorithmic_bytes_per_launch": gemv_bytes(1),
+                   "settle_ms": args.settle_ms,
+                   "settle": "the workload runs untimed for settle_ms right before its warm-up steps (steady clocks); "
+                             "extras.gemv_i4g32_M1_first_measurement_of_the_process is the same measurement without it"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_bytes,
                      "traffic_source": "hardware counters of an earlier profiled run, read from the committed summary "
                                        "profiles/gemv_i4g32_m1_config1_hbm_traffic.txt (not measured by this run)",
-                     "kernel": kernel_name, "wall_clock_us_per_step": round(wall1, 3)},
+                     "kernel": kernel_name, "host_us_per_step": round(wall1, 3)},
         "cpu_baseline": cpu,
         "parity": parity,
         "extras": extras,

@@ -103,30 +103,8 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
     const int KH = K >> 1, G = K >> 5;
     const int row = (r < pv && n0 + r < N) ? n0 + r : (n0 < N ? n0 : N - 1);
     const uint32_t wrow = (uint32_t)row * (uint32_t)KH;  // byte offset; the host checks N*K/2 < 2^31
-    const uint32_t mask_r = vgpr_const(0x000F000Fu), magic_r = vgpr_const(kBf16Magic);
-
-    // the zero block that A lanes off the diagonal (and padding activation rows) read from
-    for (int o = tid * 16; o < ZERO_BYTES; o += T * 16)
-        *reinterpret_cast<u32x4 *>(lds + C::ZERO_OFF + o) = u32x4{0, 0, 0, 0};
-
-    // A-operand address of this lane per pass: real data only on the diagonal (row 4j'+v meets k-slot
-    // group j = j') and where activation row p*MPASS + v%MPASS exists; all other lanes read zeros (stride
-    // 0 keeps them inside the zero block)
-    uint32_t a_base[MP], a_step[MP];
-#pragma unroll
-    for (int p = 0; p < MP; ++p) {
-        const int v = lane & 3;
-        const bool act = (((lane & 15) >> 2) == j) && (p * MPASS + (v % MPASS) < M);
-        a_base[p] = act ? (uint32_t)(p * C::PASS + ks * S * 1024 + 64 * j + 16 * v) : (uint32_t)C::ZERO_OFF;
-        a_step[p] = act ? 1024u : 0u;
-    }
-
-    f32x4 acc[MP];
-#pragma unroll
-    for (int p = 0; p < MP; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // scale tile of this wave: P rows x 32*HP groups; lane -> (row, 8-group piece) for the single load
-    uint8_t *sct = lds + C::SC_OFF + wave * C::SC_WAVE;
     int srow_l[C::SC_NL], spiece[C::SC_NL], srow[C::SC_NL];  // piece lane + 64*l; pieces beyond P rows repeat a valid row
 #pragma unroll
     for (int l = 0; l < C::SC_NL; ++l) {
@@ -139,13 +117,27 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
     // [M,N] block of y: the split-K form for matrices with too few rows to fill the chip
     const int kbeg = blockIdx.y * kspan, kend = (kbeg + kspan < K) ? kbeg + kspan : K;
     y += (size_t)blockIdx.y * M * N;
-    for (int kc0 = kbeg; kc0 < kend; kc0 += KC) {
+
+    // ---- the requests of a chunk.  Every wave issues, in this order, its activation loads, ONE load for its tile of
+    // scales and its first D weight loads, all before the first wait (memory returns in order, so what is needed first
+    // is asked for first).  For the first chunk this is the first thing the kernel does: only the addresses above stand
+    // between the wave's start and its requests, and everything else the kernel sets up (operand addresses, the zero
+    // block, constants) is computed while they are on their way - the wave's first weights are asked for some 0.7 us
+    // earlier than when that set-up came first (about 250 vector instructions on SIMDs shared by two waves).
+    u32x4 xr[MP][XI];
+    f32x4 gr[XG ? XI : 1][4];  // XG: 8 gate and 8 up values per piece
+    f32x4 nr[XN ? 12 : 1];     // XN: residual (2), norm weight (2), up to four delta vectors (8)
+    static_assert(!XN || (M == 1 && MP == 1 && KC / 8 <= T), "the norm-folding mode stages one piece per thread");
+    const bool stager = !XN || tid < KC / 8;  // XN in a workgroup of more than KC/8 threads: the first KC/8 stage
+    u32x4 sv[C::SC_NL];
+    u32x4 w[S];
+    int kc0 = kbeg;
+    auto issue_w = [&](int i) {  // steps c = S*ks + i of the chunk at kc0; the lane takes group (c*HP + h)*4 + j
+        const int g = (kc0 >> 5) + ((S * ks + i) * HP + h) * 4 + j;
+        w[i] = load_nt_b128(wp + (wrow + (uint32_t)(g < G ? g : 0) * 16u));
+    };
+    auto request = [&]() {
         // 1. activation loads FIRST.  Piece `it` = tid + T*q of pass p: row m = it / 512, i8 = it % 512.
-        u32x4 xr[MP][XI];
-        f32x4 gr[XG ? XI : 1][4];  // XG: 8 gate and 8 up values per piece
-        f32x4 nr[XN ? 12 : 1];     // XN: residual (2), norm weight (2), up to four delta vectors (8)
-        static_assert(!XN || (M == 1 && MP == 1 && KC / 8 <= T), "the norm-folding mode stages one piece per thread");
-        const bool stager = !XN || tid < KC / 8;  // XN in a workgroup of more than KC/8 threads: the first KC/8 stage
 #pragma unroll
         for (int p = 0; p < MP; ++p)
 #pragma unroll
@@ -181,28 +173,47 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
                     xr[p][q] = *reinterpret_cast<const u32x4 *>(x + (k < K ? (size_t)(p * MPASS + m) * K + k : 0));
                 }
             }
-
         // 2. the wave's scale tile in one load.  Needs G % 8 == 0 (16-byte aligned pieces), checked on the host.
-        u32x4 sv[C::SC_NL];
 #pragma unroll
         for (int l = 0; l < C::SC_NL; ++l) {
             const int gs = (kc0 >> 5) + ks * S * 4 * HP + spiece[l] * 8;
             sv[l] = *reinterpret_cast<const u32x4 *>(sc + ((size_t)srow[l] * G + (gs < G ? gs : 0)));
             if (gs >= G) sv[l] = u32x4{0, 0, 0, 0};
         }
-
-        // 3. the wave's weight loads for the chunk: steps c = 8*ks + i, lane takes group (c*HP + h)*4 + j
-        //    Only the first D are issued now; step i issues load i+D once its own data has arrived, so a
-        //    wave's requests are spread over the stream and its last data meets one step of work, not S.
-        u32x4 w[S];
-        auto issue_w = [&](int i) {
-            const int g = (kc0 >> 5) + ((S * ks + i) * HP + h) * 4 + j;
-            w[i] = load_nt_b128(wp + (wrow + (uint32_t)(g < G ? g : 0) * 16u));
-        };
+        // 3. the wave's weight loads for the chunk.  Only the first D are issued now; step i issues load i+D once its
+        //    own data has arrived, so a wave's requests are spread over the stream and its last data meets one step of
+        //    work, not S.
 #pragma unroll
         for (int i = 0; i < (D < S ? D : S); ++i) issue_w(i);
         __builtin_amdgcn_sched_barrier(0);  // every load above is issued before anything below may wait
+    };
+    request();
 
+    const uint32_t mask_r = vgpr_const(0x000F000Fu), magic_r = vgpr_const(kBf16Magic);
+
+    // the zero block that A lanes off the diagonal (and padding activation rows) read from
+    for (int o = tid * 16; o < ZERO_BYTES; o += T * 16)
+        *reinterpret_cast<u32x4 *>(lds + C::ZERO_OFF + o) = u32x4{0, 0, 0, 0};
+
+    // A-operand address of this lane per pass: real data only on the diagonal (row 4j'+v meets k-slot
+    // group j = j') and where activation row p*MPASS + v%MPASS exists; all other lanes read zeros (stride
+    // 0 keeps them inside the zero block)
+    uint32_t a_base[MP], a_step[MP];
+#pragma unroll
+    for (int p = 0; p < MP; ++p) {
+        const int v = lane & 3;
+        const bool act = (((lane & 15) >> 2) == j) && (p * MPASS + (v % MPASS) < M);
+        a_base[p] = act ? (uint32_t)(p * C::PASS + ks * S * 1024 + 64 * j + 16 * v) : (uint32_t)C::ZERO_OFF;
+        a_step[p] = act ? 1024u : 0u;
+    }
+
+    f32x4 acc[MP];
+#pragma unroll
+    for (int p = 0; p < MP; ++p) acc[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    uint8_t *sct = lds + C::SC_OFF + wave * C::SC_WAVE;  // the wave's scale tile in LDS
+
+    for (;;) {  // one pass per chunk of KC; the norm-folding mode has a single chunk by contract
         // 4. stage the activations: 16-byte pieces (8 k) -> [c][t][j][v], paired for the unpack order, and
         //    the C operands -136 * (sum of the group's 32 activations)
         float nv[8];
@@ -316,6 +327,9 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
                 a_addr[p] += a_step[p];
             }
         }
+        kc0 += KC;
+        if (XN || kc0 >= kend) break;
+        request();
     }
 
     // 6a. One activation row and one wave per row block (KS = 1): everything a row's sum consists of sits in this wave -
