@@ -454,18 +454,7 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(S == 
     const int KH = K >> 1, G = K >> 5;
     const int row = (r < pv && n0 + r < N) ? n0 + r : (n0 < N ? n0 : N - 1);
     const uint32_t wrow = (uint32_t)row * (uint32_t)KH;
-    const uint32_t mask_r = vgpr_const(0x000F000Fu), magic_r = vgpr_const(kBf16Magic);
 
-    for (int o = tid * 16; o < C::ZERO_SPAN; o += T * 16) *reinterpret_cast<u32x4 *>(lds + C::ZERO_OFF + o) = u32x4{0, 0, 0, 0};
-
-    // A operand: lane (i = lane & 15, j) is row 8g + m with g = i >> 3, m = i & 7
-    const bool a_live = ((nl >> 3) == (j >> 1)) && ((nl & 7) < M);
-    const uint32_t a_base = a_live ? (uint32_t)(ks * S * 2048 + (j >> 1) * 256 + (j & 1) * 128 + (nl & 7) * 16) : (uint32_t)C::ZERO_OFF;
-    const uint32_t a_step = a_live ? 2048u : 0u;
-
-    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    uint8_t *sct = lds + C::SC_OFF + wave * C::SC_WAVE;
     int srow_l[C::SC_NL], spiece[C::SC_NL], srow[C::SC_NL];
 #pragma unroll
     for (int l = 0; l < C::SC_NL; ++l) {
@@ -486,9 +475,17 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(S == 
         c = rest >> 2;
     };
 
-    for (int kc0 = 0; kc0 < K; kc0 += KC) {
+    // the requests of a chunk, as in the kernel above: asked for before anything else is set up
+    u32x4 xr[XI];
+    u32x4 sv[C::SC_NL];
+    u32x4 w[S];
+    int kc0 = 0;
+    auto issue_w = [&](int i) {
+        const int gg = (kc0 >> 5) + (S * ks + i) * 4 + j;
+        w[i] = load_nt_b128(wp + (wrow + (uint32_t)(gg < G ? gg : 0) * 16u));
+    };
+    auto request = [&]() {
         // 1. activation loads first
-        u32x4 xr[XI];
 #pragma unroll
         for (int q = 0; q < XI; ++q) {
             int t, m, c, pr, g;
@@ -498,7 +495,6 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(S == 
             if (m < M && k < K) xr[q] = *reinterpret_cast<const u32x4 *>(x + (size_t)m * K + k);
         }
         // 2. the wave's scale tile
-        u32x4 sv[C::SC_NL];
 #pragma unroll
         for (int l = 0; l < C::SC_NL; ++l) {
             const int gs = (kc0 >> 5) + ks * S * 4 + spiece[l] * 8;
@@ -506,15 +502,26 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(S == 
             if (gs >= G) sv[l] = u32x4{0, 0, 0, 0};
         }
         // 3. the first D weight loads
-        u32x4 w[S];
-        auto issue_w = [&](int i) {
-            const int gg = (kc0 >> 5) + (S * ks + i) * 4 + j;
-            w[i] = load_nt_b128(wp + (wrow + (uint32_t)(gg < G ? gg : 0) * 16u));
-        };
 #pragma unroll
         for (int i = 0; i < (D < S ? D : S); ++i) issue_w(i);
         __builtin_amdgcn_sched_barrier(0);
+    };
+    request();
 
+    const uint32_t mask_r = vgpr_const(0x000F000Fu), magic_r = vgpr_const(kBf16Magic);
+
+    for (int o = tid * 16; o < C::ZERO_SPAN; o += T * 16) *reinterpret_cast<u32x4 *>(lds + C::ZERO_OFF + o) = u32x4{0, 0, 0, 0};
+
+    // A operand: lane (i = lane & 15, j) is row 8g + m with g = i >> 3, m = i & 7
+    const bool a_live = ((nl >> 3) == (j >> 1)) && ((nl & 7) < M);
+    const uint32_t a_base = a_live ? (uint32_t)(ks * S * 2048 + (j >> 1) * 256 + (j & 1) * 128 + (nl & 7) * 16) : (uint32_t)C::ZERO_OFF;
+    const uint32_t a_step = a_live ? 2048u : 0u;
+
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    uint8_t *sct = lds + C::SC_OFF + wave * C::SC_WAVE;
+
+    for (;;) {
         // 4. stage the activations
         __syncthreads();  // the previous chunk's operand reads (or the zero fill) are done
 #pragma unroll
@@ -574,6 +581,9 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(S == 
             }
             a_addr += a_step;
         }
+        kc0 += KC;
+        if (kc0 >= K) break;
+        request();
     }
 
     // 6. fold the two scale-group halves and the K-slices
@@ -634,7 +644,8 @@ struct GemvRows16Cfg {
 };
 
 template <int S, int RBW, int D, int KC>
-__global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(RBW == 2 ? 2 : 4))) void gemv_i4g32_mfma_rows16_kernel(
+// (two waves per SIMD at most: a workgroup's operands take 68 KB or more of LDS, so a wave may use 256 registers)
+__global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(2))) void gemv_i4g32_mfma_rows16_kernel(
     const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
     float *__restrict__ y, int M, int N, int K, int pv) {
     typedef GemvRows16Cfg<S, RBW, KC> C;
@@ -648,6 +659,47 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(RBW =
     const int KH = K >> 1, G = K >> 5;
     const int row = (r < pv && n0 + r < N) ? n0 + r : (n0 < N ? n0 : N - 1);
     const uint32_t wrow = (uint32_t)row * (uint32_t)KH;
+
+    int srow_l[C::SC_NL], spiece[C::SC_NL], srow[C::SC_NL];
+#pragma unroll
+    for (int l = 0; l < C::SC_NL; ++l) {
+        srow_l[l] = (lane + 64 * l) / C::SC_PPR;
+        spiece[l] = (lane + 64 * l) % C::SC_PPR;
+        srow[l] = (srow_l[l] < pv && n0 + srow_l[l] < N) ? n0 + srow_l[l] : (n0 < N ? n0 : N - 1);
+    }
+
+    // the requests of a chunk, as in the kernels above: asked for before anything else is set up
+    u32x4 xr[XI];
+    u32x4 sv[C::SC_NL];
+    u32x4 w[S];
+    int kc0 = 0;
+    auto issue_w = [&](int i) {
+        const int gg = (kc0 >> 5) + (S * ks + i) * 4 + j;
+        w[i] = load_nt_b128(wp + (wrow + (uint32_t)(gg < G ? gg : 0) * 16u));
+    };
+    auto request = [&]() {
+        // 1. activation loads first.  Piece it = tid + T*q: word it % 4 of its scale group, activation row
+        //    it / 4 % 16, chunk-local group it / 64: a wave stores 1 KiB of contiguous LDS.
+#pragma unroll
+        for (int q = 0; q < XI; ++q) {
+            const int it = tid + T * q, m = (it >> 2) & 15, k = kc0 + 32 * (it >> 6) + 8 * (it & 3);
+            xr[q] = u32x4{0, 0, 0, 0};
+            if (m < M && k < K) xr[q] = *reinterpret_cast<const u32x4 *>(x + (size_t)m * K + k);
+        }
+        // 2. the wave's scale tile
+#pragma unroll
+        for (int l = 0; l < C::SC_NL; ++l) {
+            const int gs = (kc0 >> 5) + ks * S * 4 + spiece[l] * 8;
+            sv[l] = *reinterpret_cast<const u32x4 *>(sc + ((size_t)srow[l] * G + (gs < G ? gs : 0)));
+            if (gs >= G) sv[l] = u32x4{0, 0, 0, 0};
+        }
+        // 3. the first D weight loads
+#pragma unroll
+        for (int i = 0; i < (D < S ? D : S); ++i) issue_w(i);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    request();
+
     const uint32_t mask_r = vgpr_const(0x000F000Fu), magic_r = vgpr_const(kBf16Magic);
 
     for (int o = tid * 16; o < C::ZERO_SPAN; o += T * 16) *reinterpret_cast<u32x4 *>(lds + C::ZERO_OFF + o) = u32x4{0, 0, 0, 0};
@@ -659,42 +711,8 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(RBW =
     f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
 
     uint8_t *sct = lds + C::SC_OFF + wave * C::SC_WAVE;
-    int srow_l[C::SC_NL], spiece[C::SC_NL], srow[C::SC_NL];
-#pragma unroll
-    for (int l = 0; l < C::SC_NL; ++l) {
-        srow_l[l] = (lane + 64 * l) / C::SC_PPR;
-        spiece[l] = (lane + 64 * l) % C::SC_PPR;
-        srow[l] = (srow_l[l] < pv && n0 + srow_l[l] < N) ? n0 + srow_l[l] : (n0 < N ? n0 : N - 1);
-    }
 
-    for (int kc0 = 0; kc0 < K; kc0 += KC) {
-        // 1. activation loads first.  Piece it = tid + T*q: word it % 4 of its scale group, activation row
-        //    it / 4 % 16, chunk-local group it / 64: a wave stores 1 KiB of contiguous LDS.
-        u32x4 xr[XI];
-#pragma unroll
-        for (int q = 0; q < XI; ++q) {
-            const int it = tid + T * q, m = (it >> 2) & 15, k = kc0 + 32 * (it >> 6) + 8 * (it & 3);
-            xr[q] = u32x4{0, 0, 0, 0};
-            if (m < M && k < K) xr[q] = *reinterpret_cast<const u32x4 *>(x + (size_t)m * K + k);
-        }
-        // 2. the wave's scale tile
-        u32x4 sv[C::SC_NL];
-#pragma unroll
-        for (int l = 0; l < C::SC_NL; ++l) {
-            const int gs = (kc0 >> 5) + ks * S * 4 + spiece[l] * 8;
-            sv[l] = *reinterpret_cast<const u32x4 *>(sc + ((size_t)srow[l] * G + (gs < G ? gs : 0)));
-            if (gs >= G) sv[l] = u32x4{0, 0, 0, 0};
-        }
-        // 3. the first D weight loads
-        u32x4 w[S];
-        auto issue_w = [&](int i) {
-            const int gg = (kc0 >> 5) + (S * ks + i) * 4 + j;
-            w[i] = load_nt_b128(wp + (wrow + (uint32_t)(gg < G ? gg : 0) * 16u));
-        };
-#pragma unroll
-        for (int i = 0; i < (D < S ? D : S); ++i) issue_w(i);
-        __builtin_amdgcn_sched_barrier(0);
-
+    for (;;) {
         // 4. stage the activations
         __syncthreads();  // the previous chunk's operand reads (or the zero fill) are done
 #pragma unroll
@@ -752,6 +770,9 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(RBW =
             }
             a_addr += a_step;
         }
+        kc0 += KC;
+        if (kc0 >= K) break;
+        request();
     }
 
     // 6. fold the K-slices
