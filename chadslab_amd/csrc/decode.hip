@@ -324,24 +324,42 @@ __global__ __launch_bounds__(256) void rope_table_kernel(float *__restrict__ tab
     table[2 * i + 1] = sn;
 }
 
-// Sum over each 32-lane half of the wave; valid in lanes 16..31 and 48..63 (data-parallel primitives only: a
-// cross-lane read through LDS costs a wait each, and there are 160 of these reductions per workgroup).
-__device__ __forceinline__ float half_wave_sum_hi(float v) {
-    v += dpp_f32<0x128, 0xF>(v);  // row_ror:8
-    v += dpp_f32<0x124, 0xF>(v);  // row_ror:4
-    v += dpp_f32<0x122, 0xF>(v);  // row_ror:2
-    v += dpp_f32<0x121, 0xF>(v);  // row_ror:1: every lane of a 16-lane row holds the row sum
-    v += dpp_f32<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
-    return v;
+// Eight fp32 values as two MFMA operands of eight bf16 each: `hi` holds the values cut off after 16 bits (exact), `lo`
+// what is left, cut off the same way, so hi + lo carries 16 mantissa bits of every value - more than the bf16 K and V
+// rows they are multiplied with.  Element e sits in half-word e.
+__device__ __forceinline__ void split_bf16x8(const f32x4 a, const f32x4 b, bf16x8 &hi, bf16x8 &lo) {
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    uint32_t h[4], l[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const uint32_t u0 = __float_as_uint(v[2 * e]), u1 = __float_as_uint(v[2 * e + 1]);
+        h[e] = __builtin_amdgcn_perm(u1, u0, 0x07060302u);  // the two high half-words
+        const float r0 = v[2 * e] - __uint_as_float(u0 & 0xFFFF0000u), r1 = v[2 * e + 1] - __uint_as_float(u1 & 0xFFFF0000u);
+        l[e] = __builtin_amdgcn_perm(__float_as_uint(r1), __float_as_uint(r0), 0x07060302u);
+    }
+    __builtin_memcpy(&hi, h, 16);
+    __builtin_memcpy(&lo, l, 16);
 }
 
 // Workgroup b: positions [32b, 32b+32).  qkv fp32 = [hq*dh | dh | dh] straight from the projection.  Every
 // workgroup rotates q itself (table lookup): thread (head, 8-column piece) rotates its piece once and the rotated q
-// goes through LDS, so a thread issues 8 loads for q instead of 36; the V slice is fetched with 16-byte loads and
-// read by columns from LDS.  The workgroup that owns position pos also rotates k, writes row pos of both caches and
-// puts the new rows into LDS instead of reading them back.  Partials as attn_mqa_partial_kernel;
-// attn_mqa_combine_kernel follows.  (Letting the last workgroup to finish do the combination in the same launch
-// was tried and lost: one workgroup pulling every partial through one CU took longer than a second launch.)
+// goes through LDS.  The workgroup that owns position pos also rotates k, writes row pos of both caches and puts the
+// new rows into LDS instead of reading them back.  Partials as attn_mqa_partial_kernel.
+//
+// Both products run on the matrix cores (v_mfma_f32_16x16x32_bf16; as dot products and column sums in the vector
+// units they took 1.5 us each of a kernel that lasted 5):
+//   scores  D[position][head] = sum_d K[position][d] * q[head][d].  A = K rows: lane (i = lane % 16, g = lane / 16)
+//           holds the 16 bytes K[16*blk + i][32*st + 8g .. +7], which is what it loads from the cache - no staging.
+//           B = q: lane (head = lane % 16, g) holds q[head][32*st + 8g .. +7] as two bf16 operands (split_bf16x8); heads
+//           8..15 are zeros.  Wave w takes the steps st = 2w, 2w+1 (64 of the 256 columns) for both blocks of 16
+//           positions: 8 MFMAs; the four waves' sums meet in LDS, where thread (head, position) picks its score up.
+//   output  D[head][column] = sum_p P[head][p] * V[p][column].  A = the probabilities (two bf16 operands again), B =
+//           V[8g .. 8g+7][16*cb + lane % 16]: eight 2-byte reads down a column of the V slice in LDS (rows padded so that
+//           the four lane groups use different banks).  Wave w takes the column blocks cb = 4w .. 4w+3: 8 MFMAs; lane
+//           (column, g < 2) then holds heads 4g .. 4g+3 of its column and stores them.
+// FULL: hq = 8 and dh = 256 (the host checks), where no operand needs a guard: the reads of a phase are then issued
+// together and its stores sit behind a single condition.
+template <bool FULL>
 __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__restrict__ qkv, const int32_t *__restrict__ pos,
                                                              const float *__restrict__ table, uint16_t *__restrict__ kc,
                                                              uint16_t *__restrict__ vc, float *__restrict__ ws,
@@ -351,12 +369,16 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
     if (p0 >= ctx) return;
     const bool own = (p - p0) < ATT_CS;  // this slice contains the new position
     float *part = ws;
-    __shared__ __attribute__((aligned(16))) float s_sc[8][ATT_CS];       // scores, then probabilities
-    __shared__ __attribute__((aligned(16))) float s_q[8][256];           // rotated q
-    __shared__ __attribute__((aligned(16))) uint16_t s_v[ATT_CS][256];   // the slice of V
-    __shared__ __attribute__((aligned(16))) uint16_t s_krow[256];        // the new (rotated) k row
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int half = dh >> 1, hw = lane >> 5, c = lane & 31, lpr = dh >> 3;
+    constexpr int VP = 264;  // half-words per row of the V slice in LDS
+    __shared__ __attribute__((aligned(16))) float s_sc[8][ATT_CS];          // probabilities
+    __shared__ __attribute__((aligned(16))) float s_q[8][256];              // rotated q
+    __shared__ __attribute__((aligned(16))) uint16_t s_v[ATT_CS][VP];       // the slice of V
+    __shared__ __attribute__((aligned(16))) uint16_t s_krow[256];           // the new (rotated) k row
+    __shared__ __attribute__((aligned(16))) float s_part[4][64][9];         // the waves' partial scores (9: bank spread)
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = dh >> 1, lpr = dh >> 3;
+    const int li = lane & 15, g = lane >> 4;
 
     // V: 16-byte pieces of the slice, piece ch = row * lpr + column piece, dealt round robin to the threads
     u32x4 vld[4];
@@ -366,15 +388,16 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
         const int pi = (p0 + row < ctx) ? p0 + row : ctx - 1;
         if (row < ATT_CS) vld[j] = *reinterpret_cast<const u32x4 *>(vc + (size_t)pi * dh + vcc * 8);
     }
-    // K: wave w owns rows 8w..8w+7 of the slice, two rows per load instruction
-    const int cc = c < lpr ? c : 0;
-    u32x4 kv[4];
+    // K: the A operands of this wave's MFMAs, kv[blk][s2] = K[16*blk + li][32*(2*wave + s2) + 8g .. +7]
+    u32x4 kv[2][2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int pl = wave * 8 + 2 * i + hw;
-        const int pi = (p0 + pl < ctx) ? p0 + pl : ctx - 1;
-        kv[i] = *reinterpret_cast<const u32x4 *>(kc + (size_t)pi * dh + cc * 8);
-    }
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            const int d0 = 32 * (2 * wave + s2) + 8 * g, pl = 16 * blk + li;
+            const int pi = (p0 + pl < ctx) ? p0 + pl : ctx - 1;
+            kv[blk][s2] = *reinterpret_cast<const u32x4 *>(kc + (size_t)pi * dh + (d0 < dh ? d0 : 0));
+        }
     // q: thread (head tid/32, piece tid%32) loads its 8 columns, the 8 columns they rotate with, and the angles
     const int qh = tid >> 5, qc = (tid & 31) < lpr ? (tid & 31) : 0;
     const bool qlive = qh < hq && (tid & 31) < lpr;
@@ -436,72 +459,46 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
         }
     }
     __syncthreads();
-    if (own) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (p0 + wave * 8 + 2 * i + hw == p) kv[i] = *reinterpret_cast<const u32x4 *>(s_krow + cc * 8);
-    }
 
-    const bool live = c < lpr;
-    const float scale = rsqrtf((float)dh);
-    // 32 partial dot products per lane (4 rows x 8 heads, index 8i + h) over the lane's 8 columns ...
-    float dots[32];
+    // scores: 2 blocks of positions x 2 steps x (hi, lo) = 8 MFMAs per wave
     {
-        f32x4 qra[8], qrb[8];
+        f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-        for (int h = 0; h < 8; ++h) {
-            qra[h] = *reinterpret_cast<const f32x4 *>(&s_q[h][cc * 8]);
-            qrb[h] = *reinterpret_cast<const f32x4 *>(&s_q[h][cc * 8 + 4]);
-        }
+        for (int s2 = 0; s2 < 2; ++s2) {
+            const int st = 2 * wave + s2, d0 = 32 * st + 8 * g;
+            if (FULL || 32 * st < dh) {  // uniform over the wave
+                const bool qok = li < 8 && (FULL || d0 < dh);  // heads 8..15 and columns past dh: zeros
+                const int dq = (FULL || d0 < dh) ? d0 : 0;
+                const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
+                f32x4 q0 = *reinterpret_cast<const f32x4 *>(&s_q[li & 7][dq]), q1 = *reinterpret_cast<const f32x4 *>(&s_q[li & 7][dq + 4]);
+                q0 = qok ? q0 : zero4;  // selected, not branched around: the reads of both steps go out together
+                q1 = qok ? q1 : zero4;
+                bf16x8 bhi, blo;
+                split_bf16x8(q0, q1, bhi, blo);
+                const u32x4 krow = *reinterpret_cast<const u32x4 *>(s_krow + dq);  // meaningful in the owner only
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t kk[4] = {kv[i].x, kv[i].y, kv[i].z, kv[i].w};
-            float k8[8];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                k8[2 * e] = live ? bf16_bits_to_f32(kk[e] & 0xFFFFu) : 0.f;
-                k8[2 * e + 1] = live ? bf16_bits_to_f32(kk[e] >> 16) : 0.f;
+                for (int blk = 0; blk < 2; ++blk) {
+                    const u32x4 kw = (own && p0 + 16 * blk + li == p) ? krow : kv[blk][s2];
+                    bf16x8 av;
+                    __builtin_memcpy(&av, &kw, 16);
+                    acc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bhi, acc[blk], 0, 0, 0);
+                    acc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, blo, acc[blk], 0, 0, 0);
+                }
             }
-#pragma unroll
-            for (int h = 0; h < 8; ++h)
-                dots[8 * i + h] = qra[h].x * k8[0] + qra[h].y * k8[1] + qra[h].z * k8[2] + qra[h].w * k8[3] + qrb[h].x * k8[4] +
-                                  qrb[h].y * k8[5] + qrb[h].z * k8[6] + qrb[h].w * k8[7];
         }
-    }
-    // ... summed over the 32 lanes of the half wave by halving: in the step with lane mask m a lane hands the half of
-    // its values whose index bit m differs from its own lane bit to lane ^ m and adds what it receives, so after
-    // five steps lane c holds the complete sum of index c: 31 exchanges instead of 32 five-step reductions.
-    // Masks 8, 2 and 1 are DPP moves (a rotation by 8 inside a 16-lane row is an exchange with lane ^ 8); 16 and 4 go
-    // through the LDS crossbar, all exchanges of a step issued before the first result is used.
-    auto halve = [&](auto m_c, auto n_c) {
-        constexpr int m = decltype(m_c)::value, n = decltype(n_c)::value;
-        const bool up = (c & m) != 0;
-        float got[n / 2];
+        // lane (head = li, g) holds positions 16*blk + 4g + e, e = 0..3
 #pragma unroll
-        for (int j = 0; j < n / 2; ++j) {
-            const float send = up ? dots[j] : dots[j + n / 2];
-            if (m == 8) got[j] = dpp_f32<0x128, 0xF>(send);
-            else if (m == 2) got[j] = dpp_f32<0x4E, 0xF>(send);
-            else if (m == 1) got[j] = dpp_f32<0xB1, 0xF>(send);
-            else got[j] = __shfl_xor(send, m, 64);
-        }
+        for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-        for (int j = 0; j < n / 2; ++j) dots[j] = (up ? dots[j + n / 2] : dots[j]) + got[j];
-    };
-    halve(std::integral_constant<int, 16>{}, std::integral_constant<int, 32>{});
-    halve(std::integral_constant<int, 8>{}, std::integral_constant<int, 16>{});
-    halve(std::integral_constant<int, 4>{}, std::integral_constant<int, 8>{});
-    halve(std::integral_constant<int, 2>{}, std::integral_constant<int, 4>{});
-    halve(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{});
-    {
-        const int i = c >> 3, h = c & 7, pl = wave * 8 + 2 * i + hw;
-        s_sc[h][pl] = (p0 + pl < ctx && h < hq) ? dots[0] * scale : -INFINITY;
+            for (int e = 0; e < 4; ++e) s_part[wave][lane][blk * 4 + e] = acc[blk][e];
     }
     __syncthreads();
     {
-        // softmax of the slice: thread -> (head tid/32, position tid%32)
+        // thread -> (head tid/32, position tid%32): its score from the four waves' parts, then the softmax of the slice
         const int h = tid >> 5, i = tid & 31;
-        const float s = s_sc[h][i];
+        const int src = 16 * ((i & 15) >> 2) + h, idx = (i >> 4) * 4 + (i & 3);
+        const float dot = (s_part[0][src][idx] + s_part[1][src][idx]) + (s_part[2][src][idx] + s_part[3][src][idx]);
+        const float s = (p0 + i < ctx && h < hq) ? dot * rsqrtf((float)dh) : -INFINITY;
         // over the 32 positions: rotations inside the 16-lane rows (DPP), then one exchange between the two rows
         float mx = s;
         mx = fmaxf(mx, dpp_f32<0x128, 0xF>(mx));  // row_ror:8
@@ -524,23 +521,41 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
         }
     }
     __syncthreads();
-    // V: thread t owns column t of every row of the slice
-    const int col = tid < dh ? tid : dh - 1;
-    float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // output: 4 column blocks x (hi, lo) = 8 MFMAs per wave
+    {
+        const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
+        f32x4 p0v = *reinterpret_cast<const f32x4 *>(&s_sc[li & 7][8 * g]), p1v = *reinterpret_cast<const f32x4 *>(&s_sc[li & 7][8 * g + 4]);
+        p0v = li < 8 ? p0v : zero4;  // rows 8..15 of A are zeros
+        p1v = li < 8 ? p1v : zero4;
+        bf16x8 ahi, alo;
+        split_bf16x8(p0v, p1v, ahi, alo);
+        // all the wave's column reads first, then its MFMAs, then its stores behind one condition
+        uint32_t bw[4][4];
 #pragma unroll
-    for (int i = 0; i < ATT_CS; i += 4) {
-        const float v0 = bf16_bits_to_f32(s_v[i][col]), v1 = bf16_bits_to_f32(s_v[i + 1][col]),
-                    v2 = bf16_bits_to_f32(s_v[i + 2][col]), v3 = bf16_bits_to_f32(s_v[i + 3][col]);
+        for (int c4 = 0; c4 < 4; ++c4) {
+            const int cb = 4 * wave + c4, col = (FULL || 16 * cb < dh) ? 16 * cb + li : 0;  // past dh: any valid column
 #pragma unroll
-        for (int h = 0; h < 8; ++h) {
-            const f32x4 p4 = *reinterpret_cast<const f32x4 *>(&s_sc[h][i]);
-            o[h] += p4.x * v0 + p4.y * v1 + p4.z * v2 + p4.w * v3;
+            for (int e = 0; e < 4; ++e)
+                bw[c4][e] = (uint32_t)s_v[8 * g + 2 * e][col] | ((uint32_t)s_v[8 * g + 2 * e + 1][col] << 16);
         }
-    }
-    if (tid < dh) {
+        f32x4 d[4];
 #pragma unroll
-        for (int h = 0; h < 8; ++h)
-            if (h < hq) part[((size_t)blockIdx.x * hq + h) * (dh + 2) + 2 + tid] = o[h];
+        for (int c4 = 0; c4 < 4; ++c4) {
+            bf16x8 bv;
+            __builtin_memcpy(&bv, bw[c4], 16);
+            d[c4] = f32x4{0.f, 0.f, 0.f, 0.f};
+            d[c4] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi, bv, d[c4], 0, 0, 0);
+            d[c4] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo, bv, d[c4], 0, 0, 0);
+        }
+        if (g < 2) {  // heads 4g .. 4g+3 of column 16*cb + li
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) {
+                const int cb = 4 * wave + c4, col = 16 * cb + li;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (FULL || (16 * cb < dh && 4 * g + e < hq)) part[((size_t)blockIdx.x * hq + 4 * g + e) * (dh + 2) + 2 + col] = d[c4][e];
+            }
+        }
     }
 }
 
@@ -816,7 +831,10 @@ int rope_table_launch(float *table, int dh, int max_ctx, float base, hipStream_t
 int attn_mqa_fused_launch(const float *qkv, const int32_t *pos, const float *table, uint16_t *kc, uint16_t *vc, float *ws,
                           uint16_t *out, int hq, int dh, int max_ctx, hipStream_t st) {
     const int nb = (max_ctx + ATT_CS - 1) / ATT_CS;
-    hipLaunchKernelGGL(attn_mqa_fused_kernel, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, out, hq, dh, max_ctx);
+    if (hq == 8 && dh == 256)
+        hipLaunchKernelGGL(attn_mqa_fused_kernel<true>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, out, hq, dh, max_ctx);
+    else
+        hipLaunchKernelGGL(attn_mqa_fused_kernel<false>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, out, hq, dh, max_ctx);
     hipLaunchKernelGGL(attn_mqa_combine_kernel, dim3(hq, (dh + 63) / 64), dim3(256), 0, st, ws, pos, out, hq, dh, max_ctx);
     return hip_check(hipGetLastError(), "attn_mqa_fused launch");
 }
@@ -828,8 +846,12 @@ bool attn_mqa_fused_oproj_ok(int hq, int dh) { return dh == 256 && hq >= 2 && hq
 int attn_mqa_fused_oproj_launch(const float *qkv, const int32_t *pos, const float *table, uint16_t *kc, uint16_t *vc, float *ws,
                                 const uint8_t *wp, const uint16_t *sc, float *y, int hq, int dh, int max_ctx, int N, hipStream_t st) {
     const int nb = (max_ctx + ATT_CS - 1) / ATT_CS;
-    hipLaunchKernelGGL(attn_mqa_fused_kernel, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, (uint16_t *)nullptr, hq, dh,
-                       max_ctx);
+    if (hq == 8)  // dh = 256 here
+        hipLaunchKernelGGL(attn_mqa_fused_kernel<true>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, (uint16_t *)nullptr, hq,
+                           dh, max_ctx);
+    else
+        hipLaunchKernelGGL(attn_mqa_fused_kernel<false>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, (uint16_t *)nullptr, hq,
+                           dh, max_ctx);
     // 64 rows per workgroup up to 4096 rows (hq/2 * N/64 workgroups: 128 for a 2048-row matrix), 128 beyond
     if (N <= 4096)
         hipLaunchKernelGGL((attn_combine_oproj_kernel<1>), dim3(hq / 2, (N + 63) / 64), dim3(1024), 0, st, ws, pos, wp, sc, y, hq, max_ctx, N);
