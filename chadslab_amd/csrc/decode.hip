@@ -363,11 +363,22 @@ template <bool FULL>
 __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__restrict__ qkv, const int32_t *__restrict__ pos,
                                                              const float *__restrict__ table, uint16_t *__restrict__ kc,
                                                              uint16_t *__restrict__ vc, float *__restrict__ ws,
-                                                             uint16_t *__restrict__ out, int hq, int dh, int max_ctx) {
-    const int p = min(max(pos[0], 0), max_ctx - 1), ctx = p + 1;
+                                                             int max_ctx, int hq_arg, int dh_arg) {
+    // (the first 14 dwords of arguments arrive in registers with the wave: everything the full instance uses)
+    const int hq = FULL ? 8 : hq_arg, dh = FULL ? 256 : dh_arg;  // constants in the full instance: no divisions by dh / 8
     const int p0 = blockIdx.x * ATT_CS;
-    if (p0 >= ctx) return;
-    const bool own = (p - p0) < ATT_CS;  // this slice contains the new position
+    const int pos_raw = pos[0];  // asked for at once, waited for as late as possible
+    // The position comes from device memory, half a microsecond away.  The full instance does not wait for it before
+    // asking for its K and V rows and q: rows are clamped to the cache instead of to the context (rows past the
+    // context then hold whatever the cache holds: their scores are masked by selection, their V rows zeroed on the way
+    // into LDS), and a workgroup past the context leaves once its requests are in LDS - which is why the host picks this
+    // instance only for caches of up to 8192 rows (at most 8 MB of such reads per launch).
+    int p = 0, ctx = 0;
+    if (!FULL) {
+        p = min(max(pos_raw, 0), max_ctx - 1), ctx = p + 1;
+        if (p0 >= ctx) return;
+    }
+    const int lim = FULL ? max_ctx : ctx;  // rows below lim may be read
     float *part = ws;
     constexpr int VP = 264;  // half-words per row of the V slice in LDS
     __shared__ __attribute__((aligned(16))) float s_sc[8][ATT_CS];          // probabilities
@@ -384,9 +395,9 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
     u32x4 vld[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int ch = tid + 256 * j, row = ch / lpr, vcc = ch % lpr;
-        const int pi = (p0 + row < ctx) ? p0 + row : ctx - 1;
-        if (row < ATT_CS) vld[j] = *reinterpret_cast<const u32x4 *>(vc + (size_t)pi * dh + vcc * 8);
+        const int ch = tid + 256 * j, row = ch / lpr, vcc = ch % lpr;  // rows past the slice (short dh): loaded, not used
+        const int pi = (p0 + row < lim) ? p0 + row : lim - 1;
+        vld[j] = *reinterpret_cast<const u32x4 *>(vc + (size_t)pi * dh + vcc * 8);
     }
     // K: the A operands of this wave's MFMAs, kv[blk][s2] = K[16*blk + li][32*(2*wave + s2) + 8g .. +7]
     u32x4 kv[2][2];
@@ -395,7 +406,7 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
             const int d0 = 32 * (2 * wave + s2) + 8 * g, pl = 16 * blk + li;
-            const int pi = (p0 + pl < ctx) ? p0 + pl : ctx - 1;
+            const int pi = (p0 + pl < lim) ? p0 + pl : lim - 1;
             kv[blk][s2] = *reinterpret_cast<const u32x4 *>(kc + (size_t)pi * dh + (d0 < dh ? d0 : 0));
         }
     // q: thread (head tid/32, piece tid%32) loads its 8 columns, the 8 columns they rotate with, and the angles
@@ -407,6 +418,13 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
     const float *qrow = qkv + (size_t)(qh < hq ? qh : 0) * dh;
     const f32x4 qa = *reinterpret_cast<const f32x4 *>(qrow + colq), qb = *reinterpret_cast<const f32x4 *>(qrow + colq + 4);
     const f32x4 pa = *reinterpret_cast<const f32x4 *>(qrow + colp), pb = *reinterpret_cast<const f32x4 *>(qrow + colp + 4);
+    if (FULL) {
+        // The requests above go out before the position is waited for.  A workgroup past the context leaves only behind
+        // the first barrier: an exit here would make the compiler move those requests behind it, where they are needed.
+        __builtin_amdgcn_sched_barrier(0);
+        p = min(max(pos_raw, 0), max_ctx - 1), ctx = p + 1;
+    }
+    const bool own = p0 < ctx && (p - p0) < ATT_CS;  // this slice contains the new position
     const float *tp = table + ((size_t)p * half + jt) * 2;
     const f32x4 t0 = *reinterpret_cast<const f32x4 *>(tp), t1 = *reinterpret_cast<const f32x4 *>(tp + 4),
                 t2 = *reinterpret_cast<const f32x4 *>(tp + 8), t3 = *reinterpret_cast<const f32x4 *>(tp + 12);
@@ -442,7 +460,8 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int ch = tid + 256 * j, row = ch / lpr, vcc = ch % lpr;
-        if (row < ATT_CS && !(own && p0 + row == p)) *reinterpret_cast<u32x4 *>(&s_v[row][vcc * 8]) = vld[j];
+        if (row < ATT_CS && !(own && p0 + row == p))
+            *reinterpret_cast<u32x4 *>(&s_v[row][vcc * 8]) = (!FULL || p0 + row < ctx) ? vld[j] : u32x4{0, 0, 0, 0};
     }
     if (own) {
         if (tid < half) {
@@ -459,6 +478,7 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
         }
     }
     __syncthreads();
+    if (FULL && p0 >= ctx) return;  // uniform over the workgroup
 
     // scores: 2 blocks of positions x 2 steps x (hi, lo) = 8 MFMAs per wave
     {
@@ -831,10 +851,10 @@ int rope_table_launch(float *table, int dh, int max_ctx, float base, hipStream_t
 int attn_mqa_fused_launch(const float *qkv, const int32_t *pos, const float *table, uint16_t *kc, uint16_t *vc, float *ws,
                           uint16_t *out, int hq, int dh, int max_ctx, hipStream_t st) {
     const int nb = (max_ctx + ATT_CS - 1) / ATT_CS;
-    if (hq == 8 && dh == 256)
-        hipLaunchKernelGGL(attn_mqa_fused_kernel<true>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, out, hq, dh, max_ctx);
+    if (hq == 8 && dh == 256 && max_ctx <= 8192)
+        hipLaunchKernelGGL(attn_mqa_fused_kernel<true>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, max_ctx, hq, dh);
     else
-        hipLaunchKernelGGL(attn_mqa_fused_kernel<false>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, out, hq, dh, max_ctx);
+        hipLaunchKernelGGL(attn_mqa_fused_kernel<false>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, max_ctx, hq, dh);
     hipLaunchKernelGGL(attn_mqa_combine_kernel, dim3(hq, (dh + 63) / 64), dim3(256), 0, st, ws, pos, out, hq, dh, max_ctx);
     return hip_check(hipGetLastError(), "attn_mqa_fused launch");
 }
@@ -846,12 +866,10 @@ bool attn_mqa_fused_oproj_ok(int hq, int dh) { return dh == 256 && hq >= 2 && hq
 int attn_mqa_fused_oproj_launch(const float *qkv, const int32_t *pos, const float *table, uint16_t *kc, uint16_t *vc, float *ws,
                                 const uint8_t *wp, const uint16_t *sc, float *y, int hq, int dh, int max_ctx, int N, hipStream_t st) {
     const int nb = (max_ctx + ATT_CS - 1) / ATT_CS;
-    if (hq == 8)  // dh = 256 here
-        hipLaunchKernelGGL(attn_mqa_fused_kernel<true>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, (uint16_t *)nullptr, hq,
-                           dh, max_ctx);
+    if (hq == 8 && max_ctx <= 8192)  // dh = 256 here
+        hipLaunchKernelGGL(attn_mqa_fused_kernel<true>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, max_ctx, hq, dh);
     else
-        hipLaunchKernelGGL(attn_mqa_fused_kernel<false>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, (uint16_t *)nullptr, hq,
-                           dh, max_ctx);
+        hipLaunchKernelGGL(attn_mqa_fused_kernel<false>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, max_ctx, hq, dh);
     // 64 rows per workgroup up to 4096 rows (hq/2 * N/64 workgroups: 128 for a 2048-row matrix), 128 beyond
     if (N <= 4096)
         hipLaunchKernelGGL((attn_combine_oproj_kernel<1>), dim3(hq / 2, (N + 63) / 64), dim3(1024), 0, st, ws, pos, wp, sc, y, hq, max_ctx, N);

@@ -349,6 +349,34 @@ def test_attn_fused_oproj_refuses_shapes_it_does_not_cover(lib):
                                                             16, stream()), "attn fused oproj")
 
 
+@pytest.mark.parametrize("hq,dh,pos,max_ctx", [(8, 256, 40, 4096), (8, 256, 2047, 4096), (8, 256, 0, 64), (4, 64, 40, 200), (8, 256, 40, 16384)])
+def test_attn_fused_never_lets_rows_past_the_context_in(lib, hq, dh, pos, max_ctx):
+    """Cache rows behind the current position hold NaN: the result must be what it is with zeros there (the kernel for
+    8 heads of 256 reads such rows before it knows the position and has to mask them; the general one never reads them)."""
+    r = rng(5 * hq + dh + pos)
+    qkv = r.standard_normal((hq + 2) * dh).astype(np.float32)
+    kc = O.f32_to_bf16(r.standard_normal((max_ctx, dh)).astype(np.float32))
+    vc = O.f32_to_bf16(r.standard_normal((max_ctx, dh)).astype(np.float32))
+    tq, tp = dev(qkv), torch.tensor([pos], dtype=torch.int32, device=DEV)
+    table = torch.zeros(max_ctx * dh, dtype=torch.float32, device=DEV)
+    chk(lib.chadq_rope_table(table.data_ptr(), dh, max_ctx, 10000.0, stream()), "table")
+    outs = []
+    for fill in (0x0000, 0x7FC0, 0x7F80):  # zeros, NaN, +inf behind the context
+        k2, v2 = kc.copy(), vc.copy()
+        k2[pos + 1:] = fill
+        v2[pos + 1:] = fill
+        tk, tv = bf16_tensor(k2.reshape(-1)), bf16_tensor(v2.reshape(-1))
+        ws = torch.zeros(lib.chadq_attn_decode_mqa_fused_workspace_floats(hq, dh, max_ctx), dtype=torch.float32, device=DEV)
+        out = torch.zeros(hq * dh, dtype=torch.bfloat16, device=DEV)
+        chk(lib.chadq_attn_decode_mqa_fused(tq.data_ptr(), tp.data_ptr(), table.data_ptr(), tk.data_ptr(), tv.data_ptr(),
+                                            ws.data_ptr(), out.data_ptr(), hq, dh, max_ctx, stream()), "attn fused")
+        torch.cuda.synchronize()
+        outs.append(bits(out).copy())
+        assert np.array_equal(bits(tk).reshape(max_ctx, dh)[pos + 1:], k2[pos + 1:])  # and never written
+    assert np.isfinite(O.bf16_to_f32(outs[0])).all()
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
 def test_rope_table_matches_the_rotation(lib):
     dh, ctx = 64, 300
     table = torch.zeros(ctx * dh, dtype=torch.float32, device=DEV)
