@@ -106,6 +106,10 @@ __device__ __forceinline__ void expert_body(const uint16_t *__restrict__ xa, con
         const int rr = (4 * i + wave) * 8 + (lane >> 3), rc = rr < rows ? rr : rows - 1;
         const size_t srow = rowidx ? (size_t)rowidx[m0 + rc] : (size_t)(m0 + rc);  // gate/up: the token of the expert's row
         asrc[i] = (uint32_t)((srow * K + (((lane & 7) ^ (rr & 7)) << 3)) * 2);
+        // A row past the tile is requested beyond the descriptor's range: the copy then delivers zeros.  Its products are
+        // never stored either way, but the matrix cores run at the clock their power allows, and a multiplier fed zeros
+        // draws less: a quarter of the rows of a typical routing are such padding.
+        if (rr >= rows) asrc[i] = 0x80000000u;
     }
     // fragment read offsets: row mb*32 + nl, piece kq*4 + j lives in slot (kq*4 + j) ^ (nl & 7)
     uint32_t ard[4];
