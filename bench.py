@@ -31,6 +31,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16
 N_COPIES = 12
 SEG = 48                     # launches per captured graph
+DEC_STEPS = 1                 # decode steps per captured graph (config 4): several per graph save nothing in a queue of replays
 
 
 def profile_figures():
@@ -506,14 +507,14 @@ def main():
                 dec.vcache[li].normal_()
             dec.token.fill_(5)
             dec.pos.fill_(2040)
-            dec.capture()
-            settle(lambda i: dec.graph.replay())  # positions 2040 .. about 2105 (max_ctx 4096); then back to the start
+            dec.capture(DEC_STEPS)
+            settle(lambda i: dec.graph.replay())  # positions 2040 .. about 2110 (max_ctx 4096); then back to the start
             dec.pos.fill_(2040)
-            for _ in range(8):
+            for _ in range(8 // DEC_STEPS):
                 dec.graph.replay()
             a4, b4 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             a4.record(stream)
-            for _ in range(n_dec):
+            for _ in range(n_dec // DEC_STEPS):
                 dec.graph.replay()
             b4.record(stream)
             torch.cuda.synchronize()
@@ -524,7 +525,8 @@ def main():
         extras["decode_step_config4"] = {"us_per_token": round(us4, 1), "tokens_per_s": round(1e6 / us4, 1),
                                          "bytes_per_token": wbytes + kvbytes, "GBps": round((wbytes + kvbytes) / us4 * 1e-3, 1),
                                          "frac_hbm_peak": round((wbytes + kvbytes) / us4 * 1e-3 / HBM_PEAK_GBS, 4),
-                                         "context": "2048..2111", "launch": "one HIP graph per token"}
+                                         "context": "2048..2111",
+                                         "launch": "one HIP graph per %d tokens (the token passes from step to step in device memory)" % DEC_STEPS}
         del dec
         # the same step ending in a draw from the 50 most likely tokens instead of the argmax (the uniform number stays
         # fixed during the replays: the draw's cost does not depend on it)
@@ -536,14 +538,14 @@ def main():
             dec.token.fill_(5)
             dec.pos.fill_(2040)
             dec.set_sampling(50, 1.0, 1004)
-            dec.capture()
+            dec.capture(DEC_STEPS)
             settle(lambda i: dec.graph.replay())
             dec.pos.fill_(2040)
-            for _ in range(8):
+            for _ in range(8 // DEC_STEPS):
                 dec.graph.replay()
             a4, b4 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             a4.record(stream)
-            for _ in range(n_dec):
+            for _ in range(n_dec // DEC_STEPS):
                 dec.graph.replay()
             b4.record(stream)
             torch.cuda.synchronize()

@@ -135,6 +135,8 @@ class QuantDecoder:
         self.kcache = [z(c.max_ctx * c.dh, bf16) for _ in range(c.n_layers)]
         self.vcache = [z(c.max_ctx * c.dh, bf16) for _ in range(c.n_layers)]
         self.graph = None
+        self.graph_steps = 1        # tokens per replay of the captured graph
+        self.ring = None            # the tokens between the steps of one replay (capture(steps > 1))
 
     # ---- single launches -------------------------------------------------------------------------------
     def _s(self):
@@ -150,13 +152,19 @@ class QuantDecoder:
                                                    w.data_ptr(), self.xn.data_ptr(), self.cfg.d, self.cfg.eps, self._s()),
                    "chadq_add_rmsnorm_bf16")
 
-    def step(self, trace: Optional[list] = None) -> None:
+    def step(self, trace: Optional[list] = None, token_in=None, token_out=None, u=None) -> None:
         """One token: reads token/pos from device memory, leaves the next token and pos+1 there.  The caller keeps
         pos below max_ctx (feed() and generate() check it on the host; the kernels only clamp for memory safety).
         trace (eager launches only, for parity checks): receives a copy of the fp32 residual vector entering every
-        layer, then of the one entering the final norm (n_layers + 1 tensors)."""
+        layer, then of the one entering the final norm (n_layers + 1 tensors).
+        token_in / token_out / u (one-element device tensors; default self.token, self.token, self.u[:1]): where the
+        step reads its token, leaves the next one and finds its uniform number - the steps of a multi-step graph
+        hand their tokens on through a ring instead of through self.token."""
         c, lib, s = self.cfg, self.lib, self._s()
-        _lib.check(lib.chadq_embed_i4g32(self.token.data_ptr(), self.w["emb"].packed.data_ptr(), self.w["emb"].scale.data_ptr(),
+        token_in = self.token if token_in is None else token_in
+        token_out = self.token if token_out is None else token_out
+        u = self.u[:1] if u is None else u
+        _lib.check(lib.chadq_embed_i4g32(token_in.data_ptr(), self.w["emb"].packed.data_ptr(), self.w["emb"].scale.data_ptr(),
                                          self.x.data_ptr(), c.d, c.vocab, s), "chadq_embed_i4g32")
         pending = None
         for li, L in enumerate(self.w["layers"]):
@@ -220,12 +228,12 @@ class QuantDecoder:
             trace.append(self.x.clone())
         self._gemv(self.xn, self.w["emb"], self.logits)
         if self.sampling is None:
-            _lib.check(lib.chadq_argmax_f32(self.logits.data_ptr(), c.vocab, self.scratch.data_ptr(), self.token.data_ptr(),
+            _lib.check(lib.chadq_argmax_f32(self.logits.data_ptr(), c.vocab, self.scratch.data_ptr(), token_out.data_ptr(),
                                             self.pos.data_ptr(), 1, s), "chadq_argmax_f32")
         else:
             k, temperature = self.sampling
-            _lib.check(lib.chadq_sample_topk_f32(self.logits.data_ptr(), c.vocab, k, temperature, self.u.data_ptr(),
-                                                 self.sample_ws.data_ptr(), self.token.data_ptr(), self.pos.data_ptr(), 1, s),
+            _lib.check(lib.chadq_sample_topk_f32(self.logits.data_ptr(), c.vocab, k, temperature, u.data_ptr(),
+                                                 self.sample_ws.data_ptr(), token_out.data_ptr(), self.pos.data_ptr(), 1, s),
                        "chadq_sample_topk_f32")
 
     def set_sampling(self, top_k: int = 0, temperature: float = 1.0, seed: int = 0) -> None:
@@ -238,19 +246,34 @@ class QuantDecoder:
         self.sampling = (int(top_k), float(temperature)) if top_k > 0 else None
         self.rng.manual_seed(seed)
 
-    def capture(self) -> None:
-        """Captures step() in a HIP graph (after one eager warm-up step whose effects are undone)."""
+    def _steps(self, k: int) -> None:
+        """k consecutive steps; the token goes from one to the next through self.ring, in and out through self.token."""
+        for j in range(k):
+            self.step(token_in=self.token if j == 0 else self.ring[j:j + 1],
+                      token_out=self.token if j == k - 1 else self.ring[j + 1:j + 2], u=self.u[j:j + 1])
+
+    def capture(self, steps: int = 1) -> None:
+        """Captures `steps` consecutive step() calls in one HIP graph (after an eager warm-up run whose effects are
+        undone).  A replay then produces `steps` tokens: replaying a graph costs about 8 us over its nodes, once per
+        replay.  The tokens of a replay are self.ring[1 : steps] followed by self.token; with sampling, step j of a
+        replay draws with self.u[j].  feed() needs a one-step graph (or none): it sets the token before every step."""
+        if steps < 1 or steps > 64:
+            raise ValueError("1 to 64 steps per graph")
+        self.graph_steps = steps
+        self.ring = torch.zeros(steps + 1, dtype=torch.int32, device=self.dev)
+        if self.u.numel() < steps:
+            self.u = torch.zeros(steps, dtype=torch.float32, device=self.dev)
         tok, pos = self.token.clone(), self.pos.clone()
         st = torch.cuda.Stream()
         st.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(st):
-            self.step()
+            self._steps(steps)
             torch.cuda.synchronize()
             self.token.copy_(tok)
             self.pos.copy_(pos)
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=st):
-                self.step()
+                self._steps(steps)
             self.token.copy_(tok)
             self.pos.copy_(pos)
         torch.cuda.current_stream().wait_stream(st)
@@ -278,7 +301,7 @@ class QuantDecoder:
             self.token.fill_(int(t))  # overrides the token the previous step proposed
             if self.sampling is not None:
                 self.u.uniform_(0.0, 1.0, generator=self.rng)
-            if self.graph is not None:
+            if self.graph is not None and self.graph_steps == 1:
                 self.graph.replay()
             else:
                 self.step()
@@ -291,12 +314,16 @@ class QuantDecoder:
         self.token.fill_(first_token)
         self.pos.fill_(pos)
         out = []
-        for _ in range(n):
+        k = self.graph_steps if self.graph is not None else 1
+        while len(out) < n:
             if self.sampling is not None:
                 self.u.uniform_(0.0, 1.0, generator=self.rng)  # eager, stream-ordered before the step or the replay
-            if self.graph is not None:
+            if self.graph is not None and n - len(out) >= k:
                 self.graph.replay()
-            else:
+                if k > 1:
+                    out.extend(int(t) for t in torch.cat((self.ring[1:k], self.token)).tolist())
+                    continue
+            else:  # no graph, or fewer tokens left than a replay produces
                 self.step()
             out.append(int(self.token.item()))
         return out

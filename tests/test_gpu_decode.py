@@ -650,6 +650,27 @@ def test_decoder_feed_then_generate_continues_the_same_sequence():
     assert b.generate(nxt, 7, 5) == seq[7:12]
 
 
+@pytest.mark.parametrize("layers,steps", [(2, 4), (3, 3), (2, 1)])
+def test_decoder_graph_of_several_steps_produces_the_same_tokens(layers, steps):
+    """A graph that holds several consecutive steps (tokens handed on through a ring in device memory) against the same
+    steps launched one by one; also a token count that is not a multiple of the graph's, and feed() beside such a graph."""
+    from chadslab_amd.decoder import DecoderConfig, QuantDecoder
+
+    cfg = DecoderConfig(n_layers=layers, d=512, hq=4, dh=64, ffn=1024, vocab=1000, max_ctx=256)
+    m = _upload(_model(48, cfg))
+    a = QuantDecoder(cfg, m, DEV)
+    seq = a.generate(5, 0, 20)
+    b = QuantDecoder(cfg, m, DEV)
+    b.capture(steps)
+    assert b.generate(5, 0, 14) == seq[:14]     # 14 = full replays plus a remainder of single steps
+    assert int(b.pos.item()) == 14
+    nxt = b.feed([5] + seq[:6], 0)               # feed sets the token before every step: one step at a time
+    assert nxt == seq[6] and int(b.pos.item()) == 7
+    assert b.generate(nxt, 7, 2 * steps) == seq[7:7 + 2 * steps]
+    with pytest.raises(ValueError):
+        b.capture(0)
+
+
 def test_decoder_step_odd_layer_count_graph_replay():
     from chadslab_amd.decoder import DecoderConfig
 
