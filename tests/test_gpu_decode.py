@@ -249,7 +249,8 @@ def test_attn_decode_mqa(lib, hq, dh, pos, max_ctx):
 
 
 @pytest.mark.parametrize("hq,dh,pos,max_ctx", [(8, 256, 0, 64), (8, 256, 31, 64), (8, 256, 32, 4096), (8, 256, 2047, 4096),
-                                               (8, 256, 4095, 4096), (8, 256, 8191, 8192), (3, 64, 200, 300), (1, 16, 70, 128)])
+                                               (8, 256, 4095, 4096), (8, 256, 8191, 8192), (3, 64, 200, 300), (1, 16, 70, 128),
+                                               (8, 256, 4099, 4100), (8, 256, 77, 4100), (8, 256, 9000, 9001), (2, 256, 100, 130)])
 def test_attn_decode_mqa_fused_equals_rope_write_attend(lib, hq, dh, pos, max_ctx):
     r = rng(7 * hq + dh + pos)
     qkv = r.standard_normal((hq + 2) * dh).astype(np.float32)
