@@ -85,9 +85,16 @@ struct GemvPre {
 //     of a gated FFN and the kernel writes h[i] = bf16( gelu_tanh(gate) * up ) through `y` (as uint16_t): the GeGLU of
 //     a decoder layer folded into the projection that produces its inputs.  The tile rows in use (pv) must be even.
 template <int MT, int HP, int S, int RBW, int D, int KC, int XM = 0, int YM = 0>
+// Argument order: the first 14 dwords of a kernel's arguments arrive in registers with the wave, the rest has to be
+// fetched (and waited for) by its first instructions.  Everything a wave needs for its first requests is therefore put
+// first - a0 = x (modes 0, 1) or pre.res (mode 2), a1 = pre.delta, a2 = pre.w, pvn = pv | pre.n << 8 - and what is
+// needed late (y, pre.res_out, pre.eps) last.
 __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) void gemv_i4g32_mfma_kernel(
-    const uint16_t *__restrict__ x, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
-    float *__restrict__ y, int N, int K, int kspan, int pv, GemvPre pre) {
+    const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc, const void *__restrict__ a0, const float *__restrict__ a1,
+    const float *__restrict__ a2, int N, int K, int pvn, int kspan, float *__restrict__ y, float *__restrict__ res_out, float eps) {
+    const uint16_t *__restrict__ x = reinterpret_cast<const uint16_t *>(a0);
+    const int pv = pvn & 0xFF;
+    const GemvPre pre{reinterpret_cast<const float *>(a0), a1, a2, res_out, pvn >> 8, eps};
     constexpr bool XG = (XM == 1), XN = (XM == 2);
     typedef GemvCfg<MT, HP, S, RBW, KC> C;
     constexpr int M = MT, MP = C::MP, MPASS = C::MPASS, P = C::P, KS = C::KS, T = C::T, XI = C::XI;
@@ -845,8 +852,10 @@ static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc,
     int pv = pick_tile_rows(N, C::P, tiles_per_wg, ksplit);
     if (YM == 1 && (pv & 1)) pv = C::P;  // pairs of rows must not straddle tiles
     const int tiles = (N + pv - 1) / pv;
+    const void *a0 = (XM == 2) ? static_cast<const void *>(pre.res) : static_cast<const void *>(x);
     hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM, YM>), dim3((tiles + tiles_per_wg - 1) / tiles_per_wg, ksplit),
-                       dim3(256 * RBW), C::TOTAL, st, x, wp, sc, y, N, K, K / ksplit, pv, pre);
+                       dim3(256 * RBW), C::TOTAL, st, wp, sc, a0, pre.delta, pre.w, N, K, pv | (pre.n << 8), K / ksplit, y, pre.res_out,
+                       pre.eps);
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma launch");
 }
 
