@@ -310,6 +310,12 @@ def main():
         for m in (1, 4, 8):
             extras["gemv_i4g32"]["M%d" % m] = {"us": round(results[m][0], 3), "GBps": round(gemv_bytes(m) / results[m][0] * 1e-3, 1),
                                                "frac_hbm_peak": round(gemv_bytes(m) / results[m][0] * 1e-3 / HBM_PEAK_GBS, 4)}
+    # the same steps replayed from captured graphs (the launch form of the other measurements), for comparison
+    us_g, _, seg_g = run_steps(gemv_step(xs[1], copies, ys[1], 1), steps1, args.warmup, direct=False)
+    extras["gemv_i4g32_M1_graph_replay"] = {
+        "us": round(us_g, 3), "GBps": round(gemv_bytes(1) / us_g * 1e-3, 1),
+        "note": "the headline's %d steps as replays of captured graphs of %d launches, settled like it: a replay costs "
+                "about 8 us of its own, which a 20-step region shows and a 960-step region does not" % (steps1, seg_g)}
     extras["gemv_i4g32_M1_first_measurement_of_the_process"] = {
         "us": round(first_m1[0], 3), "GBps": round(gemv_bytes(1) / first_m1[0] * 1e-3, 1),
         "note": "the same %d steps after %d warm-up steps and no settling phase, on a GPU that was idle until then" % (first_m1[2], args.warmup)}
