@@ -261,6 +261,9 @@ size_t chadq_attn_decode_mqa_fused_workspace_floats(int hq, int dh, int max_ctx)
  * kernel: rotates q and k of qkv (angles from rope_table), writes row pos[0] of both caches, attends over rows
  * 0..pos[0] and writes out bf16 [hq*dh].  qkv fp32 = [hq*dh | dh | dh].
  * hq <= 8, dh <= 256 and a multiple of 16, max_ctx <= 65536; qkv, rope_table and kcache 16-byte aligned.
+ * Both caches must be readable over all max_ctx rows: for hq = 8, dh = 256 and max_ctx <= 8192 the kernel asks for its
+ * rows before it has read pos[0], clamped to the cache only; rows behind pos[0] never reach a result (whatever they
+ * hold, NaN included) and are never written.
  */
 int chadq_attn_decode_mqa_fused(const float *qkv, const int32_t *pos, const float *rope_table, uint16_t *kcache_bf16,
                                 uint16_t *vcache_bf16, float *workspace, uint16_t *out_bf16, int hq, int dh, int max_ctx,
