@@ -286,7 +286,8 @@ def test_attn_decode_mqa_fused_equals_rope_write_attend(lib, hq, dh, pos, max_ct
 
 @pytest.mark.parametrize("hq,pos,max_ctx,n", [(8, 0, 64, 2048), (8, 31, 64, 2048), (8, 32, 4096, 2048), (8, 2047, 4096, 2048),
                                               (8, 2048, 4096, 2048), (8, 2111, 4096, 2048), (8, 4095, 4096, 2048),
-                                              (8, 8191, 8192, 2048), (2, 70, 128, 100), (4, 300, 512, 4100), (6, 129, 256, 65)])
+                                              (8, 8191, 8192, 2048), (2, 70, 128, 100), (4, 300, 512, 4100), (6, 129, 256, 65),
+                                              (8, 9000, 9001, 2048), (8, 100, 4100, 300)])
 def test_attn_fused_oproj_equals_attention_then_projection(lib, hq, pos, max_ctx, n):
     """The output projection with the combination of the attention partials folded in, against (a) the separate calls on the
     GPU - the same bf16 attention vector through the oracle's f64 GEMV, and identical caches - and (b) the oracle end to end."""
