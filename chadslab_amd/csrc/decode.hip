@@ -363,11 +363,17 @@ template <bool FULL>
 __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__restrict__ qkv, const int32_t *__restrict__ pos,
                                                              const float *__restrict__ table, uint16_t *__restrict__ kc,
                                                              uint16_t *__restrict__ vc, float *__restrict__ ws,
-                                                             int max_ctx, int hq_arg, int dh_arg) {
-    // (the first 14 dwords of arguments arrive in registers with the wave: everything the full instance uses)
+                                                             int max_ctx, int hq_arg, int dh_arg, float *__restrict__ yz, int nz) {
+    // (the first 14 dwords of arguments arrive in registers with the wave: everything the full instance needs for its
+    // requests; yz and nz are fetched, and used only once those requests are out)
     const int hq = FULL ? 8 : hq_arg, dh = FULL ? 256 : dh_arg;  // constants in the full instance: no divisions by dh / 8
     const int p0 = blockIdx.x * ATT_CS;
     const int pos_raw = pos[0];  // asked for at once, waited for as late as possible
+    // yz[0 .. nz): accumulators of the kernel that follows this one (the output projection adds two heads' products
+    // into each); cleared here, by every workgroup whatever the context, so that they need no launch of their own
+    auto clear_yz = [&]() {
+        for (int i = blockIdx.x * 256 + threadIdx.x; i < nz; i += gridDim.x * 256) yz[i] = 0.f;
+    };
     // The position comes from device memory, half a microsecond away.  The full instance does not wait for it before
     // asking for its K and V rows and q: rows are clamped to the cache instead of to the context (rows past the
     // context then hold whatever the cache holds: their scores are masked by selection, their V rows zeroed on the way
@@ -375,6 +381,7 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
     // instance only for caches of up to 8192 rows (at most 8 MB of such reads per launch).
     int p = 0, ctx = 0;
     if (!FULL) {
+        clear_yz();
         p = min(max(pos_raw, 0), max_ctx - 1), ctx = p + 1;
         if (p0 >= ctx) return;
     }
@@ -440,6 +447,7 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
         if (tid < dh) vnew = qkv[(size_t)(hq + 1) * dh + tid];
     }
     __builtin_amdgcn_sched_barrier(0);
+    if (FULL) clear_yz();
 
     // rotate q: low columns a*cos - b*sin, high columns b*cos + a*sin, (a, b) = (low, high) element of the pair
     {
@@ -580,22 +588,28 @@ __global__ __launch_bounds__(256) void attn_mqa_fused_kernel(const float *__rest
 }
 
 // ---- the combination of the partials folded into the output projection that consumes the attention vector ----
-// y_part[hp][n] = sum over the 512 k of head pair hp of Wo[n][k] * att[k], Wo int4 group-32 [N, hq*256], att the bf16 attention
+// y_part[h / 2][n] += sum over the 256 k of head h of Wo[n][k] * att[k], Wo int4 group-32 [N, hq*256], att the bf16 attention
 // vector attn_mqa_combine_kernel would have written.  A launch less per layer: the combination has no kernel of its own,
-// every workgroup of the projection forms the 512 attention values it multiplies with for itself.
+// every workgroup of the projection forms the 256 attention values it multiplies with for itself.
 //
-// Workgroup (hp, row block): 16 waves, 64*NL weight rows.
-//   1. Wave w takes head 2*hp + (w & 1) and the slices b = (w >> 1) + 8i of each batch of 64: lane q fetches columns
-//      4q..4q+3 of those 8 slices (the rows of the workspace are 8-byte aligned only, hence the loads of that alignment)
-//      and lane b the running maximum and sum of slice b; every wave works out the factors exp(m_b - M) itself.  Batches
-//      beyond the first (contexts over 2048 positions) are folded in with the usual rescaling.  The workgroup's weight
-//      loads - one 16-byte load per lane and 4 rows: lane (r, g) holds scale group g of its row - are issued behind the
-//      first batch and land while the combination runs.
-//   2. The eight slice groups meet in LDS; thread c sums column c, divides, rounds to bf16 and stores it where the dot
-//      products want it: 16-byte pieces of 8 k in the pair order of unpack8_magic, piece t of group g at (16t + g) * 16
-//      (the 16 lanes of a row then read 256 consecutive bytes).
-//   3. dot products with v_dot2_f32_bf16 on 128+u, -136 * sum(x) per group, the lane's scale, a sum over the 16 lanes of
-//      the row.  The parts of the hq/2 head pairs are added by the consumer (the next projection's residual add).
+// What a workgroup costs is what it pulls through its compute unit before it can start: the partials of its head,
+// 64 slices * 258 floats = 66 KB per 2048 positions.  Hence one head per workgroup (hq * N/64 workgroups: 256 for a
+// 2048-row matrix) and not a pair.  The consumer adds the vectors it is given while it forms its own activation vector,
+// and every vector more costs it time, so the two heads of a pair add into one vector by hardware float atomics.  Two
+// addends on a cleared accumulator: a + b and b + a are the same float, the result does not depend on who arrives first.
+// The attention kernel in front clears the accumulators (attn_mqa_fused_kernel's yz).  y must be ordinary device memory.
+//
+// Workgroup (h, row block): 16 waves, 64*NL weight rows.
+//   1. Wave w takes the slices b = w + 16i of each batch of 64: lane q fetches columns 4q..4q+3 of those 4 slices (the
+//      rows of the workspace are 8-byte aligned only, hence the loads of that alignment) and lane b the running maximum
+//      and sum of slice b; every wave works out the factors exp(m_b - M) itself.  Batches beyond the first (contexts over
+//      2048 positions) are folded in with the usual rescaling.  The workgroup's weight loads - one 8-byte load per lane
+//      and 4 rows: lane (r, g2) holds half of a scale group of its row - are issued behind the first batch and land while
+//      the combination runs.
+//   2. The sixteen slice groups meet in LDS; thread c sums column c, divides, rounds to bf16 and stores it where the dot
+//      products want it: 16-byte pieces of 8 k in the pair order of unpack8_magic.
+//   3. dot products with v_dot2_f32_bf16 on 128+u, -136 * sum(x) per half group, the group's scale, a sum over the 16
+//      lanes of the row.
 typedef float f32x4_a8 __attribute__((ext_vector_type(4), aligned(8)));
 
 template <int NL>
@@ -606,32 +620,32 @@ __global__ __launch_bounds__(1024) void attn_combine_oproj_kernel(const float *_
     const int K = hq * dh, KH = K >> 1, G = K >> 5;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int hp = blockIdx.x, hl = wave & 1, sg = wave >> 1, h = 2 * hp + hl;
+    const int h = blockIdx.x, sg = wave;
     const int nbmax = (max_ctx + ATT_CS - 1) / ATT_CS;
-    __shared__ __attribute__((aligned(16))) float s_num[8][2 * dh];
-    __shared__ __attribute__((aligned(16))) uint8_t s_x[2 * dh * 2];
-    __shared__ float s_den[2];
+    __shared__ __attribute__((aligned(16))) float s_num[16][dh];
+    __shared__ __attribute__((aligned(16))) uint8_t s_x[dh * 2];
+    __shared__ float s_den;
 
     const int pos0 = pos[0];  // asked for first: the only load the factors of the first batch wait for besides their own
     const size_t stride = (size_t)hq * (dh + 2);
     const float *ph = part + (size_t)h * (dh + 2);
     const int bl = lane < nbmax ? lane : nbmax - 1;
     const float m0 = ph[(size_t)bl * stride], l0 = ph[(size_t)bl * stride + 1];
-    f32x4 pre[8];
+    f32x4 pre[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int b = sg + 8 * i;
+    for (int i = 0; i < 4; ++i) {
+        const int b = sg + 16 * i;
         pre[i] = *reinterpret_cast<const f32x4_a8 *>(ph + (size_t)(b < nbmax ? b : nbmax - 1) * stride + 2 + 4 * lane);
     }
-    const int r = lane >> 4, g = lane & 15;
+    const int r = lane >> 4, g2 = lane & 15;
     const int n0 = (blockIdx.y * 16 + wave) * 4 * NL;
-    u32x4 w[NL];
+    u32x2 w[NL];
     uint16_t sw[NL];
 #pragma unroll
     for (int l = 0; l < NL; ++l) {
         const int row = n0 + 4 * l + r, rowc = row < N ? row : N - 1;
-        w[l] = load_nt_b128(wp + (size_t)rowc * KH + (size_t)(hp * 16 + g) * 16);
-        sw[l] = sc[(size_t)rowc * G + hp * 16 + g];
+        w[l] = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(wp + (size_t)rowc * KH + (size_t)(h * 16 + g2) * 8));
+        sw[l] = sc[(size_t)rowc * G + h * 8 + (g2 >> 1)];
     }
     const int ctx = min(max(pos0, 0), max_ctx - 1) + 1, nb = (ctx + ATT_CS - 1) / ATT_CS;
     __builtin_amdgcn_sched_barrier(0);
@@ -642,20 +656,20 @@ __global__ __launch_bounds__(1024) void attn_combine_oproj_kernel(const float *_
     f32x4 num = {0.f, 0.f, 0.f, 0.f};
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < 4; ++i) {
         // a slice past the context holds whatever the workspace held: selected away, not multiplied by zero (and not
         // skipped by a branch, which would move its load behind the branch)
-        const int b = sg + 8 * i;
+        const int b = sg + 16 * i;
         num += lane_value(f0, b) * (b < nb ? pre[i] : zero4);
     }
     for (int base = 64; base < nb; base += 64) {
         const int b = base + lane;
         const bool in = b < nb;
         const float mb = in ? ph[(size_t)b * stride] : -INFINITY, lb = in ? ph[(size_t)b * stride + 1] : 0.f;
-        f32x4 pv[8];
+        f32x4 pv[4];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int bb = base + sg + 8 * i;  // uniform over the wave
+        for (int i = 0; i < 4; ++i) {
+            const int bb = base + sg + 16 * i;  // uniform over the wave
             pv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
             if (bb < nb) pv[i] = *reinterpret_cast<const f32x4_a8 *>(ph + (size_t)bb * stride + 2 + 4 * lane);
         }
@@ -664,29 +678,28 @@ __global__ __launch_bounds__(1024) void attn_combine_oproj_kernel(const float *_
         den = den * rs + f * lb;
         num *= rs;
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            if (base + sg + 8 * i < nb) num += lane_value(f, sg + 8 * i) * pv[i];
+        for (int i = 0; i < 4; ++i)
+            if (base + sg + 16 * i < nb) num += lane_value(f, sg + 16 * i) * pv[i];
         M = Mn;
     }
     den = wave_sum_to_lane63(den);
-    *reinterpret_cast<f32x4 *>(&s_num[sg][hl * dh + 4 * lane]) = num;
-    if (sg == 0 && lane == 63) s_den[hl] = den;
+    *reinterpret_cast<f32x4 *>(&s_num[sg][4 * lane]) = num;
+    if (sg == 0 && lane == 63) s_den = den;
     __syncthreads();
-    if (tid < 2 * dh) {
+    if (tid < dh) {
         float t = s_num[0][tid];
 #pragma unroll
-        for (int s8 = 1; s8 < 8; ++s8) t += s_num[s8][tid];
-        const int gg = tid >> 5, tt = (tid >> 3) & 3, e = tid & 7;
-        *reinterpret_cast<uint16_t *>(s_x + (tt * 16 + gg) * 16 + (e & 3) * 4 + (e >> 2) * 2) =
-            (uint16_t)f32_to_bf16_bits(t / s_den[tid >> 8]);
+        for (int s16 = 1; s16 < 16; ++s16) t += s_num[s16][tid];
+        const int e = tid & 7;  // piece tid / 8 (8 k, 16 bytes); lane (r, g2) reads pieces 2*g2 and 2*g2 + 1
+        *reinterpret_cast<uint16_t *>(s_x + (tid >> 3) * 16 + (e & 3) * 4 + (e >> 2) * 2) = (uint16_t)f32_to_bf16_bits(t / s_den);
     }
     __syncthreads();
 
-    u32x4 xv[4];
+    u32x4 xv[2];
     float sumx = 0.f;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        xv[t] = *reinterpret_cast<const u32x4 *>(s_x + (t * 16 + g) * 16);
+    for (int t = 0; t < 2; ++t) {
+        xv[t] = *reinterpret_cast<const u32x4 *>(s_x + (2 * g2 + t) * 16);
         sumx = dot2_bf16(xv[t].x, 0x3F803F80u, sumx);
         sumx = dot2_bf16(xv[t].y, 0x3F803F80u, sumx);
         sumx = dot2_bf16(xv[t].z, 0x3F803F80u, sumx);
@@ -695,10 +708,10 @@ __global__ __launch_bounds__(1024) void attn_combine_oproj_kernel(const float *_
     const uint32_t mask_r = vgpr_const(0x000F000Fu), magic_r = vgpr_const(kBf16Magic);
 #pragma unroll
     for (int l = 0; l < NL; ++l) {
-        const uint32_t ww[4] = {w[l].x, w[l].y, w[l].z, w[l].w};
+        const uint32_t ww[2] = {w[l].x, w[l].y};
         float acc = 0.f;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < 2; ++t) {
             uint32_t pw[4];
             unpack8_magic_r(ww[t], mask_r, magic_r, pw);
             acc = dot2_bf16(pw[0], xv[t].x, acc);
@@ -712,7 +725,7 @@ __global__ __launch_bounds__(1024) void attn_combine_oproj_kernel(const float *_
         v += dpp_f32<0x122, 0xF>(v);  // row_ror:2
         v += dpp_f32<0x121, 0xF>(v);  // row_ror:1: every lane of the 16-lane row holds the row's sum
         const int row = n0 + 4 * l + r;
-        if (g == 0 && row < N) y[(size_t)hp * N + row] = v;
+        if (g2 == 0 && row < N) unsafeAtomicAdd(&y[(size_t)(h >> 1) * N + row], v);
     }
 }
 
@@ -852,9 +865,9 @@ int attn_mqa_fused_launch(const float *qkv, const int32_t *pos, const float *tab
                           uint16_t *out, int hq, int dh, int max_ctx, hipStream_t st) {
     const int nb = (max_ctx + ATT_CS - 1) / ATT_CS;
     if (hq == 8 && dh == 256 && max_ctx <= 8192)
-        hipLaunchKernelGGL(attn_mqa_fused_kernel<true>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, max_ctx, hq, dh);
+        hipLaunchKernelGGL(attn_mqa_fused_kernel<true>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, max_ctx, hq, dh, (float *)nullptr, 0);
     else
-        hipLaunchKernelGGL(attn_mqa_fused_kernel<false>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, max_ctx, hq, dh);
+        hipLaunchKernelGGL(attn_mqa_fused_kernel<false>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, max_ctx, hq, dh, (float *)nullptr, 0);
     hipLaunchKernelGGL(attn_mqa_combine_kernel, dim3(hq, (dh + 63) / 64), dim3(256), 0, st, ws, pos, out, hq, dh, max_ctx);
     return hip_check(hipGetLastError(), "attn_mqa_fused launch");
 }
@@ -867,14 +880,14 @@ int attn_mqa_fused_oproj_launch(const float *qkv, const int32_t *pos, const floa
                                 const uint8_t *wp, const uint16_t *sc, float *y, int hq, int dh, int max_ctx, int N, hipStream_t st) {
     const int nb = (max_ctx + ATT_CS - 1) / ATT_CS;
     if (hq == 8 && max_ctx <= 8192)  // dh = 256 here
-        hipLaunchKernelGGL(attn_mqa_fused_kernel<true>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, max_ctx, hq, dh);
+        hipLaunchKernelGGL(attn_mqa_fused_kernel<true>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, max_ctx, hq, dh, y, (hq / 2) * N);
     else
-        hipLaunchKernelGGL(attn_mqa_fused_kernel<false>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, max_ctx, hq, dh);
-    // 64 rows per workgroup up to 4096 rows (hq/2 * N/64 workgroups: 128 for a 2048-row matrix), 128 beyond
+        hipLaunchKernelGGL(attn_mqa_fused_kernel<false>, dim3(nb), dim3(256), 0, st, qkv, pos, table, kc, vc, ws, max_ctx, hq, dh, y, (hq / 2) * N);
+    // 64 rows per workgroup up to 4096 rows (hq * N/64 workgroups: 256 for a 2048-row matrix), 128 beyond
     if (N <= 4096)
-        hipLaunchKernelGGL((attn_combine_oproj_kernel<1>), dim3(hq / 2, (N + 63) / 64), dim3(1024), 0, st, ws, pos, wp, sc, y, hq, max_ctx, N);
+        hipLaunchKernelGGL((attn_combine_oproj_kernel<1>), dim3(hq, (N + 63) / 64), dim3(1024), 0, st, ws, pos, wp, sc, y, hq, max_ctx, N);
     else
-        hipLaunchKernelGGL((attn_combine_oproj_kernel<2>), dim3(hq / 2, (N + 127) / 128), dim3(1024), 0, st, ws, pos, wp, sc, y, hq, max_ctx, N);
+        hipLaunchKernelGGL((attn_combine_oproj_kernel<2>), dim3(hq, (N + 127) / 128), dim3(1024), 0, st, ws, pos, wp, sc, y, hq, max_ctx, N);
     return hip_check(hipGetLastError(), "attn_mqa_fused_oproj launch");
 }
 

@@ -98,7 +98,7 @@ class QuantDecoder:
         self.qkv, self.q = z((c.hq + 2) * c.dh, f32), z(c.hq * c.dh, f32)
         # the combination of the attention partials folded into the o projection, which then leaves one partial vector
         # per pair of heads for the next residual add (the entry point's rules: dh = 256, an even hq; the adds that
-        # follow take up to four vectors)
+        # follow take up to four vectors; the entry point clears the vectors itself before its heads add into them)
         self.fused_oproj = c.dh == 256 and c.hq in (2, 4, 6, 8) and c.max_ctx <= 65536
         self.att, self.ao = z(c.hq * c.dh, bf16), z((c.hq // 2 if self.fused_oproj else 1) * c.d, f32)
         # the down projection has few rows and a long K: split it over K when that fills the chip better

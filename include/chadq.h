@@ -276,6 +276,9 @@ int chadq_attn_decode_mqa_fused(const float *qkv, const int32_t *pos, const floa
  * of heads: y_parts fp32 [hq/2, N] receives one partial vector per pair and the caller (or the n_delta argument of
  * chadq_gemv_i4g32_addnorm / _addnorm_geglu / chadq_add_rmsnorm_bf16) adds them, in order.  The attention vector itself
  * is rounded to bf16 as chadq_attn_decode_mqa_fused rounds it, but is not written anywhere.
+ * y_parts must be ordinary device memory (hipMalloc): the first kernel clears it, and in the second the two heads of a
+ * pair add their products into it with hardware float atomics - two addends on a cleared value, so the result is the
+ * same bits whichever arrives first.
  * dh = 256 and hq in {2, 4, 6, 8} (CHADQ_ERR_SHAPE otherwise: use the two separate calls), max_ctx <= 65536, N >= 1;
  * qkv, rope_table, kcache, workspace and wp 16-byte aligned.  Workspace as chadq_attn_decode_mqa_fused_workspace_floats.
  * The reference has no counterpart: its numpy runtime would call the attention and the projection one after the other.

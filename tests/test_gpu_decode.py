@@ -314,7 +314,8 @@ def test_attn_fused_oproj_equals_attention_then_projection(lib, hq, pos, max_ctx
     tk2, tv2 = bf16_tensor(kc.reshape(-1)), bf16_tensor(vc.reshape(-1))
     ws2 = torch.full((nws,), float("nan"), dtype=torch.float32, device=DEV)
     parts = torch.full((hq // 2, n), float("nan"), dtype=torch.float32, device=DEV)
-    for call in range(2):  # the second call finds the new row already in the cache
+    prev = None
+    for call in range(3):  # the later calls find the new row already in the cache
         chk(lib.chadq_attn_decode_mqa_fused_oproj_i4g32(tq.data_ptr(), tp.data_ptr(), table.data_ptr(), tk2.data_ptr(),
                                                         tv2.data_ptr(), ws2.data_ptr(), tw.data_ptr(), ts.data_ptr(),
                                                         parts.data_ptr(), hq, dh, max_ctx, n, stream()), "attn fused oproj")
@@ -322,6 +323,9 @@ def test_attn_fused_oproj_equals_attention_then_projection(lib, hq, pos, max_ctx
         got = parts.cpu().numpy()
         assert np.isfinite(got).all(), "call %d" % call
         assert np.array_equal(bits(tk2), bits(tk1)) and np.array_equal(bits(tv2), bits(tv1))
+        # the two heads of a pair add into one accumulator in whatever order they arrive: the same bits every time
+        assert prev is None or np.array_equal(got.view(np.uint32), prev.view(np.uint32)), "call %d" % call
+        prev = got.copy()
         # (a) per pair of heads, on the attention vector the separate kernel rounded to bf16: the two combinations may
         # round a value to neighbouring bf16 numbers, nothing more
         ab = bits(att)
