@@ -58,6 +58,9 @@ SIGNATURES = {
                                                    c_void_p]),
     "chadq_geglu_bf16": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     "chadq_argmax_f32": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "chadq_gemv_i4g32_argmax_scratch_bytes": (c_size_t, [c_int, c_int]),
+    "chadq_gemv_i4g32_argmax": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                        c_void_p, c_void_p]),
     "chadq_sample_topk_f32": (c_int, [c_void_p, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
 }
 

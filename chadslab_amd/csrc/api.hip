@@ -90,6 +90,11 @@ int attn_mqa_fused_static_launch(const float *, const int32_t *, const float *, 
                                  hipStream_t);
 int attn_mqa_fused_static_max_ctx();
 int argmax_launch(const float *, int, float *, int32_t *, int32_t *, int32_t *, int, hipStream_t);
+int argmax_embed_launch(const float *, bool, float *, int32_t *, int, int, int32_t *, int32_t *, int, const uint8_t *, const uint16_t *,
+                        float *, int, hipStream_t);
+bool gemv_i4g32_argmax_ok(const uint16_t *, int, int);
+int gemv_i4g32_argmax_launch(const uint16_t *, const uint8_t *, const uint16_t *, float *, int, int, float *, int32_t *, int *,
+                             hipStream_t);
 int sample_topk_launch(const float *, int, int, float, const float *, float *, int32_t *, int32_t *, int32_t *, int, hipStream_t);
 
 }  // namespace chadq
@@ -455,6 +460,43 @@ int chadq_argmax_f32(const float *v, int n, void *scratch, int32_t *token, int32
     float *pv = reinterpret_cast<float *>(scratch);
     int32_t *pi = reinterpret_cast<int32_t *>(pv + 256);
     return argmax_launch(v, n, pv, pi, token, pos, advance, st);
+}
+
+// candidates of the GEMV's workgroups: at least 24 rows each (four 8-row tiles that may use 6 of their rows)
+static size_t gemv_argmax_candidates(int N) {
+    const size_t wgs = ((size_t)(N + 5) / 6 + 3) / 4;
+    return wgs > 256 ? wgs : 256;
+}
+
+size_t chadq_gemv_i4g32_argmax_scratch_bytes(int N, int K) {
+    (void)K;
+    return N >= 1 ? 8 * gemv_argmax_candidates(N) : 0;
+}
+
+int chadq_gemv_i4g32_argmax(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *scale_f16, float *y, int N, int K,
+                            void *scratch, int32_t *token, int32_t *pos, int advance, float *next_x, void *stream) {
+    ENTER();
+    CHADQ_REQUIRE(N >= 1 && K >= 32 && K % 32 == 0, CHADQ_ERR_SHAPE,
+                  "chadq_gemv_i4g32_argmax: N=%d K=%d (K must be a positive multiple of 32)", N, K);
+    CHADQ_REQUIRE(x_bf16 && wp && scale_f16 && y && scratch && token && (pos || !advance), CHADQ_ERR_NULL,
+                  "chadq_gemv_i4g32_argmax: null pointer");
+    CHADQ_REQUIRE(aligned16(x_bf16) && aligned16(wp), CHADQ_ERR_ALIGN, "chadq_gemv_i4g32_argmax: x and wp must be 16-byte aligned");
+    const size_t cap = gemv_argmax_candidates(N);
+    float *pv = reinterpret_cast<float *>(scratch);
+    int32_t *pi = reinterpret_cast<int32_t *>(pv + cap);
+    if (gemv_i4g32_argmax_ok(scale_f16, N, K)) {
+        int n_cand = 0;
+        int rc = gemv_i4g32_argmax_launch(x_bf16, nullptr, scale_f16, y, N, K, pv, pi, &n_cand, st);  // the grid only
+        if (rc != 0) return rc;
+        CHADQ_REQUIRE(n_cand >= 1 && (size_t)n_cand <= cap, CHADQ_ERR_SHAPE,
+                      "chadq_gemv_i4g32_argmax: %d workgroups for %zu candidate slots", n_cand, cap);
+        rc = gemv_i4g32_argmax_launch(x_bf16, wp, scale_f16, y, N, K, pv, pi, &n_cand, st);
+        if (rc != 0) return rc;
+        return argmax_embed_launch(y, false, pv, pi, n_cand, N, token, pos, advance, wp, scale_f16, next_x, K, st);
+    }
+    const int rc = gemv_i4g32_mfma_dispatch(x_bf16, wp, scale_f16, y, 1, N, K, st);
+    if (rc != 0) return rc;
+    return argmax_embed_launch(y, true, pv, pi, 256, N, token, pos, advance, wp, scale_f16, next_x, K, st);
 }
 
 int chadq_sample_topk_f32(const float *v, int n, int k, float temperature, const float *u, void *workspace, int32_t *token,

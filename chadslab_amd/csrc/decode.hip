@@ -38,17 +38,34 @@ __device__ __forceinline__ float block_max(float v, float *scratch) {
     return t;
 }
 
-// x[d] = (u - 8) * scale of row `token` of the tied int4 table [V, d]
-__global__ __launch_bounds__(256) void embed_i4g32_kernel(const int32_t *__restrict__ token, const uint8_t *__restrict__ wp,
-                                                          const uint16_t *__restrict__ sc, float *__restrict__ x, int d, int V) {
-    const int t = min(max(token[0], 0), V - 1);  // a token outside the table must not become an address
+// x[d] = (u - 8) * scale of row t of the tied int4 table [V, d], by one workgroup.  Eight weights per thread and round
+// where the pointers allow it (one 4-byte load, one scale, two 16-byte stores), the plain loop otherwise: same values.
+__device__ __forceinline__ void embed_row(int t, const uint8_t *__restrict__ wp, const uint16_t *__restrict__ sc,
+                                          float *__restrict__ x, int d) {
     const uint8_t *row = wp + (size_t)t * (d / 2);
     const uint16_t *srow = sc + (size_t)t * (d / 32);
+    if (((reinterpret_cast<uintptr_t>(row) & 3u) | (reinterpret_cast<uintptr_t>(x) & 15u)) == 0) {
+        for (int k8 = threadIdx.x; k8 < (d >> 3); k8 += blockDim.x) {
+            const uint32_t w = *reinterpret_cast<const uint32_t *>(row + 4 * k8);
+            const float s = f16_bits_to_f32(srow[k8 >> 2]);
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = (float)((int)((w >> (4 * e)) & 15u) - 8) * s;
+            *reinterpret_cast<f32x4 *>(x + 8 * k8) = f32x4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<f32x4 *>(x + 8 * k8 + 4) = f32x4{v[4], v[5], v[6], v[7]};
+        }
+        return;
+    }
     for (int k = threadIdx.x; k < d; k += blockDim.x) {
         const uint8_t b = row[k >> 1];
         const int u = (k & 1) ? (b >> 4) : (b & 15);
         x[k] = (float)(u - 8) * f16_bits_to_f32(srow[k >> 5]);
     }
+}
+
+__global__ __launch_bounds__(256) void embed_i4g32_kernel(const int32_t *__restrict__ token, const uint8_t *__restrict__ wp,
+                                                          const uint16_t *__restrict__ sc, float *__restrict__ x, int d, int V) {
+    embed_row(min(max(token[0], 0), V - 1), wp, sc, x, d);  // a token outside the table must not become an address
 }
 
 // res += sum_j delta[j] (nd vectors of d floats, added in order), y = bf16(rmsnorm(res) * w); one workgroup.
@@ -789,25 +806,40 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(const float *__rest
     argmax_block(best, bi, pv + blockIdx.x, pi + blockIdx.x);
 }
 
+// ex != nullptr: the winner's row of the tied int4 table [n, d] is also written to ex as embed_i4g32_kernel would write
+// it - the residual vector the next decode step starts from, without a launch of its own.
 __global__ __launch_bounds__(256) void argmax_final_kernel(const float *__restrict__ pv, const int32_t *__restrict__ pi, int nb, int n,
                                                            int32_t *__restrict__ token, int32_t *__restrict__ pos,
-                                                           int advance) {
+                                                           int advance, const uint8_t *__restrict__ ewp,
+                                                           const uint16_t *__restrict__ esc, float *__restrict__ ex, int d) {
     __shared__ float fv;
     __shared__ int32_t fi;
     float best = -INFINITY;
     int bi = INT_MAX;
-    for (int i = threadIdx.x; i < nb; i += blockDim.x) {
-        const float x = pv[i];
-        const int xi = pi[i];
-        if (xi != INT_MAX && (bi == INT_MAX || x > best || (x == best && xi < bi))) {
-            best = x;
-            bi = xi;
+    for (int i0 = threadIdx.x; i0 < nb; i0 += 16 * 256) {  // 16 candidates in flight per thread: one workgroup reads them all
+        float x[16];
+        int xi[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int i = i0 + 256 * j;
+            x[j] = pv[i < nb ? i : 0];
+            xi[j] = i < nb ? pi[i] : INT_MAX;
         }
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+            if (xi[j] != INT_MAX && (bi == INT_MAX || x[j] > best || (x[j] == best && xi[j] < bi))) {
+                best = x[j];
+                bi = xi[j];
+            }
     }
     argmax_block(best, bi, &fv, &fi);
     if (threadIdx.x == 0) {
         token[0] = (fi == INT_MAX) ? 0 : min(max(fi, 0), n - 1);
         if (advance) pos[0] += 1;
+    }
+    if (ex) {
+        __syncthreads();  // fi, written by the first thread
+        embed_row((fi == INT_MAX) ? 0 : min(max(fi, 0), n - 1), ewp, esc, ex, d);
     }
 }
 
@@ -938,7 +970,20 @@ int geglu_launch(const float *gu, uint16_t *h, int F, hipStream_t st) {
 int argmax_launch(const float *v, int n, float *pv, int32_t *pi, int32_t *token, int32_t *pos, int advance, hipStream_t st) {
     const int nb = 256;
     hipLaunchKernelGGL(argmax_partial_kernel, dim3(nb), dim3(256), 0, st, v, n, pv, pi);
-    hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, st, pv, pi, nb, n, token, pos, advance);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, st, pv, pi, nb, n, token, pos, advance, (const uint8_t *)nullptr,
+                       (const uint16_t *)nullptr, (float *)nullptr, 0);
+    return hip_check(hipGetLastError(), "argmax launch");
+}
+
+// The second stage alone, over nb candidates some other kernel left (or, partial = true, both stages over the n values v),
+// with the winner's table row written to ex (ex = nullptr: not).
+int argmax_embed_launch(const float *v, bool partial, float *pv, int32_t *pi, int nb, int n, int32_t *token, int32_t *pos, int advance,
+                        const uint8_t *ewp, const uint16_t *esc, float *ex, int d, hipStream_t st) {
+    if (partial) {
+        nb = 256;
+        hipLaunchKernelGGL(argmax_partial_kernel, dim3(nb), dim3(256), 0, st, v, n, pv, pi);
+    }
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, st, pv, pi, nb, n, token, pos, advance, ewp, esc, ex, d);
     return hip_check(hipGetLastError(), "argmax launch");
 }
 

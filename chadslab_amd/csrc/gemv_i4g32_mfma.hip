@@ -84,6 +84,10 @@ struct GemvPre {
 // YM: what becomes of the sums.  0: y[m,n] fp32.  1 (M = 1): the rows come in pairs (2i, 2i+1) = (gate, up) of feature i
 //     of a gated FFN and the kernel writes h[i] = bf16( gelu_tanh(gate) * up ) through `y` (as uint16_t): the GeGLU of
 //     a decoder layer folded into the projection that produces its inputs.  The tile rows in use (pv) must be even.
+//     2 (M = 1, one wave per row block): y as for 0, and every workgroup also leaves the largest of its sums and that row's
+//     index in cand_v[blockIdx.x] / cand_i[blockIdx.x] (a1 / a2 of the kernel; lowest row among equal sums, NaN never a
+//     candidate, (-inf, INT_MAX) if the workgroup has none): the first stage of an argmax over y, so that a greedy
+//     decoder's pass over its 256000 logits needs no read of them.
 template <int MT, int HP, int S, int RBW, int D, int KC, int XM = 0, int YM = 0>
 // Argument order: the first 14 dwords of a kernel's arguments arrive in registers with the wave, the rest has to be
 // fetched (and waited for) by its first instructions.  Everything a wave needs for its first requests is therefore put
@@ -359,11 +363,41 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
             const float up = dpp_f32<0xB1, 0xF>(t);  // quad_perm [1,0,3,2]: the up row of the pair sits in the next lane
             if (lane < P && !(lane & 1) && lane + 1 < pv && nn + 1 < N)
                 reinterpret_cast<uint16_t *>(y)[nn >> 1] = (uint16_t)f32_to_bf16_bits(gelu_tanh_dev(t) * up);
+        } else if constexpr (YM == 2) {
+            const bool valid = lane < P && lane < pv && nn < N;
+            if (valid) y[nn] = t;
+            // the wave's candidate, then the workgroup's: the one place where this path meets the other waves
+            __shared__ float s_cv[4 * RBW];
+            __shared__ int32_t s_ci[4 * RBW];
+            const uint32_t gi = wave_winner<64>(valid && t == t, t, nn);
+            if (gi == 0xFFFFFFFFu) {
+                if (lane == 0) {
+                    s_cv[wave] = -INFINITY;
+                    s_ci[wave] = INT_MAX;
+                }
+            } else if (valid && (uint32_t)nn == gi) {  // one lane: rows are distinct
+                s_cv[wave] = t;
+                s_ci[wave] = nn;
+            }
+            __syncthreads();
+            if (tid == 0) {
+                float bv = s_cv[0];
+                int32_t bb = s_ci[0];
+#pragma unroll
+                for (int w2 = 1; w2 < 4 * RBW; ++w2)
+                    if (s_ci[w2] != INT_MAX && (bb == INT_MAX || s_cv[w2] > bv || (s_cv[w2] == bv && s_ci[w2] < bb))) {
+                        bv = s_cv[w2];
+                        bb = s_ci[w2];
+                    }
+                const_cast<float *>(a1)[blockIdx.x] = bv;
+                reinterpret_cast<int32_t *>(const_cast<float *>(a2))[blockIdx.x] = bb;
+            }
         } else {
             if (lane < P && lane < pv && nn < N) y[nn] = t;
         }
         return;
     }
+    static_assert(YM != 2 || (M == 1 && KS == 1 && HP >= 2), "argmax candidates: only the form whose waves fold their own sums writes them");
     // 6b. fold lane groups, K-parts and K-slices through LDS: RED[wave][lane][pass] = 4 floats
     __syncthreads();  // every wave is done with the operand area, which the partial sums now reuse
     u32x4 *red = reinterpret_cast<u32x4 *>(lds);
@@ -840,7 +874,7 @@ static int pick_tile_rows(int N, int P, int tiles_per_wg, int ksplit) {
 
 template <int MT, int HP, int S, int RBW, int D, int KC = 4096, int XM = 0, int YM = 0>
 static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K,
-                       hipStream_t st, int ksplit = 1, GemvPre pre = GemvPre{}) {
+                       hipStream_t st, int ksplit = 1, GemvPre pre = GemvPre{}, int *workgroups = nullptr) {
     typedef GemvCfg<MT, HP, S, RBW, KC> C;
     static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
     if (!attr_set.load(std::memory_order_acquire)) {
@@ -853,6 +887,8 @@ static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc,
     if (YM == 1 && (pv & 1)) pv = C::P;  // pairs of rows must not straddle tiles
     const int tiles = (N + pv - 1) / pv;
     const void *a0 = (XM == 2) ? static_cast<const void *>(pre.res) : static_cast<const void *>(x);
+    if (workgroups) *workgroups = (tiles + tiles_per_wg - 1) / tiles_per_wg;
+    if (workgroups && !wp) return 0;  // asked for the grid only
     hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM, YM>), dim3((tiles + tiles_per_wg - 1) / tiles_per_wg, ksplit),
                        dim3(256 * RBW), C::TOTAL, st, wp, sc, a0, pre.delta, pre.w, N, K, pv | (pre.n << 8), K / ksplit, y, pre.res_out,
                        pre.eps);
@@ -945,6 +981,20 @@ int gemv_i4g32_mfma_dispatch(const uint16_t *x, const uint8_t *wp, const uint16_
         if (rc != 0) return rc;
     }
     return 0;
+}
+
+// y = W x (M = 1) with the per-workgroup argmax candidates of y written beside it (YM = 2 above).  Only the shape of a
+// decoder's output table is covered: many rows, K <= 2048.  *n_cand receives the number of candidates (workgroups);
+// wp = nullptr asks for that number only.
+bool gemv_i4g32_argmax_ok(const uint16_t *sc, int N, int K) {
+    return N >= 8192 && K <= 2048 && (K & 255) == 0 && (int64_t)N * (K / 2) < ((int64_t)1 << 31) &&
+           (reinterpret_cast<uintptr_t>(sc) & 15u) == 0;
+}
+
+int gemv_i4g32_argmax_launch(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K, float *cand_v,
+                             int32_t *cand_i, int *n_cand, hipStream_t st) {
+    const GemvPre pre{nullptr, cand_v, reinterpret_cast<const float *>(cand_i), nullptr, 0, 0.f};
+    return launch_mfma<1, 2, 8, 1, 4, 2048, 0, 2>(x, wp, sc, y, N, K, st, 1, pre, n_cand);
 }
 
 // Split-K form, M = 1: part s of y_parts [ksplit, N] holds the sum over k in [s*K/ksplit, (s+1)*K/ksplit).

@@ -126,7 +126,7 @@ class QuantDecoder:
                                                  torch.cuda.current_stream().cuda_stream), "chadq_rope_table")
         else:
             self.part = z(self.lib.chadq_attn_decode_mqa_workspace_floats(c.hq, c.dh, c.max_ctx), f32)
-        self.scratch = z(512, f32)
+        self.scratch = z(max(512, self.lib.chadq_gemv_i4g32_argmax_scratch_bytes(c.vocab, c.d) // 4), f32)
         self.token, self.pos = z(1, i32), z(1, i32)
         # sampling: (top_k, temperature) or None for greedy; the uniform draw lives in device memory, refreshed per step
         self.sampling = None
@@ -152,9 +152,26 @@ class QuantDecoder:
                                                    w.data_ptr(), self.xn.data_ptr(), self.cfg.d, self.cfg.eps, self._s()),
                    "chadq_add_rmsnorm_bf16")
 
-    def step(self, trace: Optional[list] = None, token_in=None, token_out=None, u=None) -> None:
+    def embed_token(self) -> None:
+        """self.x = the table row of self.token: what a step without its own embedding launch (step(embed=False), every
+        step of a graph captured in greedy mode) expects to find.  A greedy step leaves the row of the token it chose
+        there itself; call this after writing self.token by hand (set_state() does)."""
+        c = self.cfg
+        _lib.check(self.lib.chadq_embed_i4g32(self.token.data_ptr(), self.w["emb"].packed.data_ptr(), self.w["emb"].scale.data_ptr(),
+                                              self.x.data_ptr(), c.d, c.vocab, self._s()), "chadq_embed_i4g32")
+
+    def set_state(self, token: int, pos: int) -> None:
+        """The token the next step consumes and its position, as feed() and generate() set them."""
+        self._check_range(pos, 1, (token,))
+        self.token.fill_(int(token))
+        self.pos.fill_(int(pos))
+        self.embed_token()
+
+    def step(self, trace: Optional[list] = None, token_in=None, token_out=None, u=None, embed: bool = True) -> None:
         """One token: reads token/pos from device memory, leaves the next token and pos+1 there.  The caller keeps
         pos below max_ctx (feed() and generate() check it on the host; the kernels only clamp for memory safety).
+        embed = False: self.x already holds the token's table row (embed_token(), or the greedy step before this one,
+        whose last kernel writes the row of the token it chose), and the step saves the launch that would fetch it.
         trace (eager launches only, for parity checks): receives a copy of the fp32 residual vector entering every
         layer, then of the one entering the final norm (n_layers + 1 tensors).
         token_in / token_out / u (one-element device tensors; default self.token, self.token, self.u[:1]): where the
@@ -164,8 +181,10 @@ class QuantDecoder:
         token_in = self.token if token_in is None else token_in
         token_out = self.token if token_out is None else token_out
         u = self.u[:1] if u is None else u
-        _lib.check(lib.chadq_embed_i4g32(token_in.data_ptr(), self.w["emb"].packed.data_ptr(), self.w["emb"].scale.data_ptr(),
-                                         self.x.data_ptr(), c.d, c.vocab, s), "chadq_embed_i4g32")
+        x_start = self.x  # the buffer a step starts from; the layers below may leave self.x naming the other one
+        if embed:
+            _lib.check(lib.chadq_embed_i4g32(token_in.data_ptr(), self.w["emb"].packed.data_ptr(), self.w["emb"].scale.data_ptr(),
+                                             self.x.data_ptr(), c.d, c.vocab, s), "chadq_embed_i4g32")
         pending = None
         for li, L in enumerate(self.w["layers"]):
             if self.fused_norm1:
@@ -226,15 +245,22 @@ class QuantDecoder:
         self._norm(pending, self.w["lnf"])
         if trace is not None:
             trace.append(self.x.clone())
-        self._gemv(self.xn, self.w["emb"], self.logits)
         if self.sampling is None:
-            _lib.check(lib.chadq_argmax_f32(self.logits.data_ptr(), c.vocab, self.scratch.data_ptr(), token_out.data_ptr(),
-                                            self.pos.data_ptr(), 1, s), "chadq_argmax_f32")
+            # the output table's GEMV leaves per-workgroup argmax candidates; the kernel that picks the winner also writes
+            # the winner's table row where the next step starts from
+            emb = self.w["emb"]
+            _lib.check(lib.chadq_gemv_i4g32_argmax(self.xn.data_ptr(), emb.packed.data_ptr(), emb.scale.data_ptr(),
+                                                   self.logits.data_ptr(), emb.N, emb.K, self.scratch.data_ptr(),
+                                                   token_out.data_ptr(), self.pos.data_ptr(), 1, x_start.data_ptr(), s),
+                       "chadq_gemv_i4g32_argmax")
         else:
+            self._gemv(self.xn, self.w["emb"], self.logits)
             k, temperature = self.sampling
             _lib.check(lib.chadq_sample_topk_f32(self.logits.data_ptr(), c.vocab, k, temperature, u.data_ptr(),
                                                  self.sample_ws.data_ptr(), token_out.data_ptr(), self.pos.data_ptr(), 1, s),
                        "chadq_sample_topk_f32")
+        if self.x is not x_start:  # an odd number of exchanges: the next step starts from the same buffer as this one
+            self.x, self.x2 = x_start, self.x
 
     def set_sampling(self, top_k: int = 0, temperature: float = 1.0, seed: int = 0) -> None:
         """top_k = 0: greedy (argmax).  Otherwise the next token is drawn from the top_k most likely ones at the given
@@ -246,17 +272,22 @@ class QuantDecoder:
         self.sampling = (int(top_k), float(temperature)) if top_k > 0 else None
         self.rng.manual_seed(seed)
 
-    def _steps(self, k: int) -> None:
-        """k consecutive steps; the token goes from one to the next through self.ring, in and out through self.token."""
+    def _steps(self, k: int, embed_first: bool = True) -> None:
+        """k consecutive steps; the token goes from one to the next through self.ring, in and out through self.token.
+        Greedy steps hand the next token's table row on themselves: only the first may need a launch for it."""
         for j in range(k):
             self.step(token_in=self.token if j == 0 else self.ring[j:j + 1],
-                      token_out=self.token if j == k - 1 else self.ring[j + 1:j + 2], u=self.u[j:j + 1])
+                      token_out=self.token if j == k - 1 else self.ring[j + 1:j + 2], u=self.u[j:j + 1],
+                      embed=embed_first if j == 0 else self.sampling is not None)
 
     def capture(self, steps: int = 1) -> None:
         """Captures `steps` consecutive step() calls in one HIP graph (after an eager warm-up run whose effects are
         undone).  A replay then produces `steps` tokens: replaying a graph costs about 8 us over its nodes, once per
         replay.  The tokens of a replay are self.ring[1 : steps] followed by self.token; with sampling, step j of a
-        replay draws with self.u[j].  feed() needs a one-step graph (or none): it sets the token before every step."""
+        replay draws with self.u[j].  feed() needs a one-step graph (or none): it sets the token before every step.
+        A graph captured in greedy mode holds no embedding launch: it starts from the table row in self.x, which capture()
+        itself, set_state(), feed(), generate() and every greedy step leave there; after writing self.token by hand,
+        call embed_token() before the next replay."""
         if steps < 1 or steps > 64:
             raise ValueError("1 to 64 steps per graph")
         self.graph_steps = steps
@@ -273,9 +304,10 @@ class QuantDecoder:
             self.pos.copy_(pos)
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=st):
-                self._steps(steps)
+                self._steps(steps, embed_first=self.sampling is not None)
             self.token.copy_(tok)
             self.pos.copy_(pos)
+            self.embed_token()
         torch.cuda.current_stream().wait_stream(st)
         torch.cuda.synchronize()
         self.graph = g
@@ -302,6 +334,8 @@ class QuantDecoder:
             if self.sampling is not None:
                 self.u.uniform_(0.0, 1.0, generator=self.rng)
             if self.graph is not None and self.graph_steps == 1:
+                if self.sampling is None:
+                    self.embed_token()  # a greedy graph starts from the row, and the row in place is the proposed token's
                 self.graph.replay()
             else:
                 self.step()
@@ -313,6 +347,7 @@ class QuantDecoder:
         self._check_range(pos, n, (first_token,))
         self.token.fill_(first_token)
         self.pos.fill_(pos)
+        self.embed_token()
         out = []
         k = self.graph_steps if self.graph is not None else 1
         while len(out) < n:

@@ -313,6 +313,21 @@ int chadq_geglu_bf16(const float *gu, uint16_t *h_bf16, int F, void *stream);
 int chadq_argmax_f32(const float *v, int n, void *scratch, int32_t *token, int32_t *pos, int advance, void *stream);
 
 /*
+ * A greedy decoder's last two calls and the next step's first in two launches: y = W x as chadq_gemv_i4g32 with M = 1
+ * (W the int4 group-32 output table [N, K]), token[0] = argmax of y by the rules of chadq_argmax_f32, pos[0] += 1 if
+ * advance != 0, and - next_x != NULL - next_x fp32 [K] = row token[0] of the same table, as chadq_embed_i4g32 would
+ * write it (tied input and output embeddings: the vector the next step starts from).
+ * For N >= 8192, K <= 2048 and a multiple of 256, N*K/2 < 2^31 and 16-byte aligned scales, every workgroup of the GEMV
+ * leaves the largest of its 64 sums beside y and the second launch reads those candidates, not y; other shapes run the
+ * separate kernels (same results).  scratch: chadq_gemv_i4g32_argmax_scratch_bytes(N, K) bytes.
+ * x and wp 16-byte aligned.  The reference has no counterpart: its numpy runtime would call the
+ * three operations one after the other.
+ */
+size_t chadq_gemv_i4g32_argmax_scratch_bytes(int N, int K);
+int chadq_gemv_i4g32_argmax(const uint16_t *x_bf16, const uint8_t *wp, const uint16_t *scale_f16, float *y, int N, int K,
+                            void *scratch, int32_t *token, int32_t *pos, int advance, float *next_x, void *stream);
+
+/*
  * Top-k sampling.  Candidates: the k largest of v[0..n), larger first, lower index first among equals (NaN is never
  * a candidate).  p_j = exp((v_j - v_0) / temperature) in that order; token[0] = the first candidate whose running
  * sum of p exceeds u[0] * (sum of p), u[0] in [0, 1) read from device memory at run time (so a captured graph draws

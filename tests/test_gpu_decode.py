@@ -440,6 +440,77 @@ def test_argmax_and_advance(lib, n):
     assert int(tok.item()) == int(np.argmax(v)) and int(pos.item()) == 42
 
 
+@pytest.mark.parametrize("n,k", [(256000, 2048), (8192, 256), (9001, 1024), (20000, 2048), (1000, 512), (8192, 4096), (300, 64)])
+def test_gemv_argmax_equals_gemv_then_argmax_then_embed(lib, n, k):
+    """The output table's GEMV with the argmax candidates in its epilogue and the winner's table row written by the kernel
+    that picks it, against the three separate calls: the same logits, token and row, bit for bit - with equal largest
+    logits in three different workgroups (the lowest row must win), with NaN activations (token 0) and without the row."""
+    r = rng(3 * n + k)
+    u = r.integers(0, 16, (n, k), dtype=np.uint8)
+    packed = (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8)
+    sc = r.lognormal(-5, 0.5, (n, k // 32)).astype(np.float16)
+    xb = O.f32_to_bf16(r.standard_normal((1, k)).astype(np.float32))
+    tx = bf16_tensor(xb.reshape(-1))
+    nscr = lib.chadq_gemv_i4g32_argmax_scratch_bytes(n, k)
+    assert nscr >= 2048
+
+    def separate(tp_, ts, txx):
+        y = torch.zeros(n, dtype=torch.float32, device=DEV)
+        tok = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+        scratch = torch.zeros(512, dtype=torch.float32, device=DEV)
+        row = torch.zeros(k, dtype=torch.float32, device=DEV)
+        chk(lib.chadq_gemv_i4g32(txx.data_ptr(), tp_.data_ptr(), ts.data_ptr(), y.data_ptr(), 1, n, k, stream()), "gemv")
+        chk(lib.chadq_argmax_f32(y.data_ptr(), n, scratch.data_ptr(), tok.data_ptr(), None, 0, stream()), "argmax")
+        chk(lib.chadq_embed_i4g32(tok.data_ptr(), tp_.data_ptr(), ts.data_ptr(), row.data_ptr(), k, n, stream()), "embed")
+        return y.cpu().numpy(), int(tok.item()), row.cpu().numpy()
+
+    def fused(tp_, ts, txx, with_row=True, advance=1):
+        y = torch.full((n,), float("nan"), dtype=torch.float32, device=DEV)
+        tok = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+        pos = torch.tensor([41], dtype=torch.int32, device=DEV)
+        scratch = torch.full((nscr // 4,), float("nan"), dtype=torch.float32, device=DEV)
+        row = torch.full((k,), float("nan"), dtype=torch.float32, device=DEV)
+        chk(lib.chadq_gemv_i4g32_argmax(txx.data_ptr(), tp_.data_ptr(), ts.data_ptr(), y.data_ptr(), n, k, scratch.data_ptr(),
+                                        tok.data_ptr(), pos.data_ptr() if advance else None, advance,
+                                        row.data_ptr() if with_row else None, stream()), "gemv argmax")
+        assert int(pos.item()) == 41 + advance
+        return y.cpu().numpy(), int(tok.item()), row.cpu().numpy()
+
+    def same(a, b):
+        return np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+    tp_, ts = dev(packed), dev(sc)
+    y0, t0, row0 = separate(tp_, ts, tx)
+    y1, t1, row1 = fused(tp_, ts, tx)
+    assert O.rel_l2(y0, O.qgemm_int4g32_f64(xb, packed, sc)[0]) < 1e-3
+    assert same(y1, y0) and t1 == t0 == int(np.argmax(y0)) and same(row1, row0)
+    assert same(row1, ((packed_u(packed[t1]).astype(np.float32) - 8) * np.repeat(sc[t1].astype(np.float32), 32)))
+    y2, t2, row2 = fused(tp_, ts, tx, with_row=False, advance=0)
+    assert same(y2, y0) and t2 == t0 and np.isnan(row2).all()
+    # the winning row copied to an earlier and a later row, far enough apart to sit in other workgroups
+    if n >= 300:
+        lo, hi = (t0 + n // 3) % n, (t0 + 2 * n // 3) % n
+        first = min(lo, hi, t0)
+        p2, s2 = packed.copy(), sc.copy()
+        p2[[lo, hi]], s2[[lo, hi]] = packed[t0], sc[t0]
+        tp2, ts2 = dev(p2), dev(s2)
+        ya, ta, rowa = separate(tp2, ts2, tx)
+        yb, tb, rowb = fused(tp2, ts2, tx)
+        assert ya[lo] == ya[hi] == ya[t0] == ya.max()
+        assert same(yb, ya) and ta == tb == first and same(rowb, rowa)
+    # NaN activations: every logit NaN, token 0 and its row
+    xn = xb.copy()
+    xn[0, 5] = 0x7FC0
+    yn, tn, rown = fused(tp_, ts, bf16_tensor(xn.reshape(-1)))
+    assert np.isnan(yn).all() and tn == 0
+    assert same(rown, ((packed_u(packed[0]).astype(np.float32) - 8) * np.repeat(sc[0].astype(np.float32), 32)))
+
+
+def packed_u(row):
+    """The 4-bit values of a packed row, low nibble first."""
+    return np.stack([row & 15, row >> 4], axis=-1).reshape(-1)
+
+
 def _sample_margin(v, k, temperature, u):
     """Distance of u from the nearest interval boundary of the truncated softmax (float64), as a fraction of 1."""
     idx = np.arange(v.size)[~np.isnan(v)]
@@ -675,6 +746,41 @@ def test_decoder_graph_of_several_steps_produces_the_same_tokens(layers, steps):
     assert b.generate(nxt, 7, 2 * steps) == seq[7:7 + 2 * steps]
     with pytest.raises(ValueError):
         b.capture(0)
+
+
+@pytest.mark.parametrize("layers", [2, 3])
+def test_decoder_greedy_step_hands_the_next_row_on(layers):
+    """A greedy step's last kernel writes the table row of the token it chose where the next step starts from: a step
+    without its own embedding launch must then give the same bits as one with it, eagerly and from a graph (which holds
+    no embedding launch), also after the token was set by hand (set_state / embed_token)."""
+    from chadslab_amd.decoder import DecoderConfig, QuantDecoder
+
+    cfg = DecoderConfig(n_layers=layers, d=512, hq=4, dh=64, ffn=1024, vocab=1000, max_ctx=64)
+    m = _upload(_model(49, cfg))
+    a, b, c = QuantDecoder(cfg, m, DEV), QuantDecoder(cfg, m, DEV), QuantDecoder(cfg, m, DEV)
+    for d in (a, b, c):
+        d.set_state(9, 3)
+    c.capture()  # (its warm-up run writes cache row 3 as the first replay will)
+    logits = []
+    for d, run in ((a, lambda: a.step()), (b, lambda: b.step(embed=False)), (c, lambda: c.graph.replay())):
+        seq = []
+        for _ in range(3):
+            run()
+            seq.append((d.logits.cpu().numpy().copy(), int(d.token.item()), int(d.pos.item())))
+        logits.append(seq)
+    for other in logits[1:]:
+        for (la, ta, pa), (lo, to, po) in zip(logits[0], other):
+            assert np.array_equal(la, lo) and ta == to and pa == po
+    # a token written by hand needs its row fetched before a step that does not fetch it
+    for d in (a, c):
+        d.token.fill_(77)
+        d.pos.fill_(10)
+    a.step()
+    c.embed_token()
+    c.graph.replay()
+    assert np.array_equal(a.logits.cpu().numpy(), c.logits.cpu().numpy()) and int(a.token.item()) == int(c.token.item())
+    with pytest.raises(ValueError):
+        a.set_state(cfg.vocab, 0)
 
 
 def test_decoder_step_odd_layer_count_graph_replay():
