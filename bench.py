@@ -144,7 +144,8 @@ def main():
     def run_steps(fn, steps, warmup, direct=False, do_settle=True):
         """fn(i) launches step i on the current stream.  Returns (us per step from HIP events, wall us per step,
         launches per replayed graph - 0 for plain stream launches).  direct: try run_direct first.  Graph form: the start
-        event is recorded behind one more untimed replay that is already queued, for the reason given in run_direct."""
+        event is recorded behind untimed replays (about 4 * COVER steps) that are already queued, for the reason given
+        in run_direct."""
         if direct:
             res = run_direct(fn, steps, warmup, do_settle)
             if res is not None:
@@ -170,7 +171,9 @@ def main():
             a = torch.cuda.Event(enable_timing=True)
             b = torch.cuda.Event(enable_timing=True)
             t0 = time.perf_counter()
-            graphs[seg].replay()  # untimed: keeps the GPU busy while the timed replays are submitted
+            n_cover = (4 * COVER + seg - 1) // seg  # untimed replays that keep the GPU busy while the timed ones are submitted
+            for _ in range(n_cover):
+                graphs[seg].replay()
             a.record(stream)
             for _ in range(full):
                 graphs[seg].replay()
@@ -179,7 +182,7 @@ def main():
             b.record(stream)
             torch.cuda.synchronize()
             t1 = time.perf_counter()
-        return a.elapsed_time(b) * 1000.0 / steps, (t1 - t0) * 1e6 / (steps + seg), seg
+        return a.elapsed_time(b) * 1000.0 / steps, (t1 - t0) * 1e6 / (steps + n_cover * seg), seg
 
     if args.calibration_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
