@@ -88,7 +88,7 @@ struct GemvPre {
 //     index in cand_v[blockIdx.x] / cand_i[blockIdx.x] (a1 / a2 of the kernel; lowest row among equal sums, NaN never a
 //     candidate, (-inf, INT_MAX) if the workgroup has none): the first stage of an argmax over y, so that a greedy
 //     decoder's pass over its 256000 logits needs no read of them.
-template <int MT, int HP, int S, int RBW, int D, int KC, int XM = 0, int YM = 0>
+template <int MT, int HP, int S, int RBW, int D, int KC, int XM = 0, int YM = 0, int D0 = D>
 // Argument order: the first 14 dwords of a kernel's arguments arrive in registers with the wave, the rest has to be
 // fetched (and waited for) by its first instructions.  Everything a wave needs for its first requests is therefore put
 // first - a0 = x (modes 0, 1) or pre.res (mode 2), a1 = pre.delta, a2 = pre.w, pvn = pv | pre.n << 8 - and what is
@@ -193,9 +193,11 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
         }
         // 3. the wave's weight loads for the chunk.  Only the first D are issued now; step i issues load i+D once its
         //    own data has arrived, so a wave's requests are spread over the stream and its last data meets one step of
-        //    work, not S.
+        //    work, not S.  (D0 < D: only D0 of them now, the others behind the staging barrier.  In the 16-wave
+        //    workgroups of the norm-folding mode four waves fetch what the activation vector is formed from and twelve
+        //    wait for them: every weight load those twelve put in front of the compute unit's queue delays all sixteen.)
 #pragma unroll
-        for (int i = 0; i < (D < S ? D : S); ++i) issue_w(i);
+        for (int i = 0; i < (D0 < S ? D0 : S); ++i) issue_w(i);
         __builtin_amdgcn_sched_barrier(0);  // every load above is issued before anything below may wait
     };
     request();
@@ -302,6 +304,10 @@ __global__ __launch_bounds__(256 * RBW) __attribute__((amdgpu_waves_per_eu(4))) 
                     *reinterpret_cast<float *>(lds + p * C::PASS + C::XA_BYTES + (c * 4 + jj) * 16 + vv * 4) = -kMagicBias * sum;
             }
         __syncthreads();
+        if (D0 < D) {
+#pragma unroll
+            for (int i = D0; i < (D < S ? D : S); ++i) issue_w(i);
+        }
 
         // 5. the chunk's 8 steps of this wave
         uint32_t a_addr[MP];
@@ -872,13 +878,13 @@ static int pick_tile_rows(int N, int P, int tiles_per_wg, int ksplit) {
     return best;
 }
 
-template <int MT, int HP, int S, int RBW, int D, int KC = 4096, int XM = 0, int YM = 0>
+template <int MT, int HP, int S, int RBW, int D, int KC = 4096, int XM = 0, int YM = 0, int D0 = D>
 static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y, int N, int K,
                        hipStream_t st, int ksplit = 1, GemvPre pre = GemvPre{}, int *workgroups = nullptr) {
     typedef GemvCfg<MT, HP, S, RBW, KC> C;
     static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
     if (!attr_set.load(std::memory_order_acquire)) {
-        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM, YM>),
+        CHADQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM, YM, D0>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::TOTAL));
         attr_set.store(true, std::memory_order_release);
     }
@@ -889,7 +895,7 @@ static int launch_mfma(const uint16_t *x, const uint8_t *wp, const uint16_t *sc,
     const void *a0 = (XM == 2) ? static_cast<const void *>(pre.res) : static_cast<const void *>(x);
     if (workgroups) *workgroups = (tiles + tiles_per_wg - 1) / tiles_per_wg;
     if (workgroups && !wp) return 0;  // asked for the grid only
-    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM, YM>), dim3((tiles + tiles_per_wg - 1) / tiles_per_wg, ksplit),
+    hipLaunchKernelGGL((gemv_i4g32_mfma_kernel<MT, HP, S, RBW, D, KC, XM, YM, D0>), dim3((tiles + tiles_per_wg - 1) / tiles_per_wg, ksplit),
                        dim3(256 * RBW), C::TOTAL, st, wp, sc, a0, pre.delta, pre.w, N, K, pv | (pre.n << 8), K / ksplit, y, pre.res_out,
                        pre.eps);
     return hip_check(hipGetLastError(), "gemv_i4g32_mfma launch");
@@ -1001,7 +1007,7 @@ int gemv_i4g32_argmax_launch(const uint16_t *x, const uint8_t *wp, const uint16_
 // K / ksplit must be a multiple of the 4096-wide chunk.
 int gemv_i4g32_splitk_launch(const uint16_t *x, const uint8_t *wp, const uint16_t *sc, float *y_parts, int N, int K,
                              int ksplit, hipStream_t st) {
-    return launch_mfma<1, 4, 8, 1, 3>(x, wp, sc, y_parts, N, K, st, ksplit);
+    return launch_mfma<1, 4, 8, 1, 4>(x, wp, sc, y_parts, N, K, st, ksplit);
 }
 
 // The same with x[k] = bf16( gelu_tanh(gu[k]) * gu[K + k] ) formed inside the kernel.
@@ -1016,8 +1022,9 @@ int gemv_i4g32_splitk_geglu_launch(const float *gu, const uint8_t *wp, const uin
 int gemv_i4g32_addnorm_launch(const float *res, const float *delta, int n, const float *w, float eps, float *res_out,
                               const uint8_t *wp, const uint16_t *sc, float *y, int N, int K, hipStream_t st) {
     const GemvPre pre{res, delta, w, res_out, n, eps};
-    // many rows: workgroups of 16 waves, so that a compute unit forms the activation vector once, not four times
-    if (N >= 8192) return launch_mfma<1, 2, 8, 4, 4, 2048, 2>(nullptr, wp, sc, y, N, K, st, 1, pre);
+    // many rows: workgroups of 16 waves, so that a compute unit forms the activation vector once, not four times; two
+    // weight loads per wave before the vector is formed and a prefetch distance of three behind it measured best
+    if (N >= 8192) return launch_mfma<1, 2, 8, 4, 3, 2048, 2, 0, 2>(nullptr, wp, sc, y, N, K, st, 1, pre);
     return launch_mfma<1, 4, 4, 1, 4, 2048, 2>(nullptr, wp, sc, y, N, K, st, 1, pre);
 }
 
@@ -1026,7 +1033,7 @@ int gemv_i4g32_addnorm_geglu_launch(const float *res, const float *delta, int n,
                                     const uint8_t *wp, const uint16_t *sc, uint16_t *h, int N, int K, hipStream_t st) {
     const GemvPre pre{res, delta, w, res_out, n, eps};
     float *y = reinterpret_cast<float *>(h);
-    if (N >= 8192) return launch_mfma<1, 2, 8, 4, 4, 2048, 2, 1>(nullptr, wp, sc, y, N, K, st, 1, pre);
+    if (N >= 8192) return launch_mfma<1, 2, 8, 4, 3, 2048, 2, 1, 2>(nullptr, wp, sc, y, N, K, st, 1, pre);
     return launch_mfma<1, 4, 4, 1, 4, 2048, 2, 1>(nullptr, wp, sc, y, N, K, st, 1, pre);
 }
 
